@@ -60,7 +60,12 @@ class CacheManager:
         self.paged_groups: list = []
         self.state_groups: list = []
         self.group_of_cache: dict = {}  # cache id -> ("paged" | "state", group index, index in group)
-        for cid in sorted(requests):
+        # a mixer that keeps several things has a cache per name, under the id (cache id, name)
+        self.names_of_cache: dict = {}  # cache id -> the names under which it has caches
+        for cid in requests:
+            if isinstance(cid, tuple):
+                self.names_of_cache.setdefault(cid[0], []).append(cid[1])
+        for cid in sorted(requests, key=lambda c: (c[0], str(c[1])) if isinstance(c, tuple) else (c, "")):
             req = requests[cid]
             if isinstance(req, PagedCacheRequest):
                 groups, kind = self.paged_groups, "paged"

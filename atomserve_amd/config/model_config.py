@@ -107,3 +107,182 @@ class Qwen3Config:
             "attention_bias": False,
             "torch_dtype": "bfloat16",
         }
+
+
+# ---- Dozusun ------------------------------------------------------------------------------------------
+
+
+def _need(raw: dict, key: str, where: str):
+    if not isinstance(raw, dict) or key not in raw:
+        raise ConfigError(f"config.json lacks {where}{key}")
+    return raw[key]
+
+
+@dataclass(frozen=True)
+class DozusunDelta:
+    """A gated-delta-rule mixer's sizes."""
+
+    heads: int  # value heads
+    kv_heads: int  # query/key heads
+    dim: int  # width of a query/key head
+    vdim: int  # width of a value head
+    conv: int  # taps of the short convolutions
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "DozusunDelta":
+        return cls(*(int(_need(raw, k, where)) for k in ("heads", "kv_heads", "dim", "vdim", "conv")))
+
+
+@dataclass(frozen=True)
+class DozusunSideBySide:
+    """An attention (left) and a gated linear recurrence (right) reading the same input."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    window: int  # keys a position sees, itself included; 0: all
+    scale: float  # multiplies q.k
+    left_scale: float
+    width: int  # channels of the recurrence
+    blocks: int  # diagonal blocks of its gates
+    conv: int
+    right_scale: float
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "DozusunSideBySide":
+        left, right = _need(raw, "left", where), _need(raw, "right", where)
+        mask = left.get("mask") or {}
+        return cls(
+            heads=int(_need(left, "heads", where + "left.")),
+            kv_heads=int(_need(left, "kv_heads", where + "left.")),
+            dim=int(_need(left, "dim", where + "left.")),
+            vdim=int(_need(left, "vdim", where + "left.")),
+            window=int(mask.get("size", 0)),
+            scale=float(_need(left, "scale", where + "left.")),
+            left_scale=float(_need(raw, "left_scale", where)),
+            width=int(_need(right, "width", where + "right.")),
+            blocks=int(_need(right, "blocks", where + "right.")),
+            conv=int(_need(right, "conv", where + "right.")),
+            right_scale=float(_need(raw, "right_scale", where)),
+        )
+
+
+@dataclass(frozen=True)
+class DozusunFeedForward:
+    kind: str  # "dense" or "moe"
+    ff: int  # width inside the feed-forward (of one expert for "moe")
+    experts: int = 0
+    top: int = 0
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "DozusunFeedForward":
+        kind = _need(raw, "kind", where)
+        if kind == "dense":
+            return cls("dense", int(_need(raw, "ff", where)))
+        if kind == "moe":
+            router = _need(raw, "router", where)
+            return cls("moe", int(_need(_need(raw, "expert", where), "ff", where + "expert.")),
+                       int(_need(router, "experts", where + "router.")), int(_need(router, "top", where + "router.")))  # fmt: skip
+        raise ConfigError(f"{where}kind={kind!r} is not supported ('dense' or 'moe')")
+
+
+@dataclass(frozen=True)
+class DozusunLayer:
+    type: str  # "delta" or "parallel"
+    mixer: object  # DozusunDelta or DozusunSideBySide
+    mlp: object  # DozusunFeedForward or None
+
+
+@dataclass(frozen=True)
+class DozusunConfig:
+    """A Dozusun decoder: layers of two kinds of mixers with dense or table-routed feed-forwards, both parts of
+    a layer reading the same stream; a stretch of layers may run several times in a row."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: tuple  # of DozusunLayer
+    loop_start: int = 0  # layers loop_start .. loop_stop - 1 run loop_times times in a row
+    loop_stop: int = 0
+    loop_times: int = 1
+
+    architecture = "Dozusun"
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "DozusunConfig":
+        _require(raw, ["vocab", "width", "layers", "norm"])
+        layers = []
+        for i, entry in enumerate(raw["layers"]):
+            where = f"layers[{i}]."
+            kind = _need(entry, "type", where)
+            if kind == "delta":
+                mixer = DozusunDelta.from_dict(_need(entry, "mixer", where), where + "mixer.")
+            elif kind == "parallel":
+                mixer = DozusunSideBySide.from_dict(_need(entry, "mixer", where), where + "mixer.")
+            else:
+                raise ConfigError(f"{where}type={kind!r} is not supported ('delta' or 'parallel')")
+            mlp = entry.get("mlp")
+            layers.append(DozusunLayer(kind, mixer, None if mlp is None else DozusunFeedForward.from_dict(mlp, where + "mlp.")))
+        loop = raw.get("loop") or {}
+        cfg = cls(
+            vocab_size=int(raw["vocab"]),
+            hidden_size=int(raw["width"]),
+            norm_eps=float(_need(raw["norm"], "eps", "norm.")),
+            layers=tuple(layers),
+            loop_start=int(loop.get("start", 0)),
+            loop_stop=int(loop.get("stop", 0)),
+            loop_times=int(loop.get("times", 1)),
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size < 1 or self.hidden_size < 1 or not self.layers:
+            raise ConfigError("vocab, width and the number of layers must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        if not 0 <= self.loop_start <= self.loop_stop <= len(self.layers) or self.loop_times < 1:
+            raise ConfigError(f"loop {self.loop_start}:{self.loop_stop} x {self.loop_times} does not fit {len(self.layers)} layers")
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            if min(m.heads, m.kv_heads, m.dim, m.vdim, m.conv) < 1 or m.heads % m.kv_heads:
+                raise ConfigError(f"layers[{i}]: head counts and sizes must be positive, heads a multiple of kv_heads")
+            if layer.type == "parallel" and (m.width < 1 or m.blocks < 1 or m.width % m.blocks or m.window < 0):
+                raise ConfigError(f"layers[{i}]: width must divide into blocks, and a window is not negative")
+            f = layer.mlp
+            if f is not None and (f.ff < 1 or (f.kind == "moe" and not 1 <= f.top <= f.experts)):
+                raise ConfigError(f"layers[{i}].mlp: sizes must be positive and top at most the number of experts")
+
+    def run_order(self) -> list:
+        """Indices of the layers in the order they run."""
+        n = len(self.layers)
+        inside = list(range(self.loop_start, self.loop_stop))
+        return list(range(self.loop_start)) + inside * self.loop_times + list(range(self.loop_stop, n))
+
+    def to_dict(self) -> dict:
+        """The config.json that `from_dict` reads back to this object."""
+        layers = []
+        for layer in self.layers:
+            m = layer.mixer
+            if layer.type == "delta":
+                mixer = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim, "conv": m.conv}
+            else:
+                left = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim, "scale": m.scale}
+                if m.window:
+                    left["mask"] = {"size": m.window}
+                mixer = {"left": left, "left_scale": m.left_scale, "right_scale": m.right_scale,
+                         "right": {"width": m.width, "blocks": m.blocks, "conv": m.conv}}  # fmt: skip
+            f = layer.mlp
+            if f is None:
+                mlp = None
+            elif f.kind == "dense":
+                mlp = {"kind": "dense", "ff": f.ff}
+            else:
+                mlp = {"kind": "moe", "expert": {"ff": f.ff}, "router": {"experts": f.experts, "top": f.top}}
+            layers.append({"type": layer.type, "mixer": mixer, "mlp": mlp})
+        raw = {"architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+               "norm": {"eps": self.norm_eps}, "layers": layers}  # fmt: skip
+        if self.loop_times > 1 or self.loop_stop > self.loop_start:
+            raw["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
+        return raw

@@ -20,8 +20,10 @@ class Architecture:
     parse_config:   raw config.json dict -> typed configuration (validates)
     build_plan:     typed configuration -> parts.plan.ModelPlan (layers as data)
     checkpoint_map: typed configuration -> {plan tensor name: [checkpoint names to stack]}
-    checkpoint_shapes: typed configuration -> {checkpoint name: (shape, "matrix" | "vector")},
-                    in the order in which random weights are drawn
+    checkpoint_shapes: typed configuration -> {checkpoint name: (shape, role)}, in the order in which
+                    random weights are drawn; roles: "matrix", "vector" (gains around 1), "bias" and
+                    "log_rate" (small values around 0), "expert_table:<experts>" (int32 rows of distinct
+                    expert numbers)
     ignored:        typed configuration -> checkpoint names that may be present and unused
     """
 
@@ -52,6 +54,8 @@ def architecture_for(raw: dict) -> Architecture:
     """The registered architecture that config.json names, or a ConfigError listing what is."""
     _load_builtin()
     names = raw.get("architectures") or []
+    if not names and isinstance(raw.get("architecture"), str):  # some configurations name theirs in the singular
+        names = [raw["architecture"]]
     if len(names) != 1 or names[0] not in _ARCHITECTURES:
         raise ConfigError(
             f"atomserve_amd only supports {', '.join(sorted(_ARCHITECTURES))}; "
@@ -73,4 +77,5 @@ def load_model_config(model_dir: str) -> tuple[Architecture, Any]:
 
 def _load_builtin() -> None:
     # Imported lazily: the model modules import parts, which import this package.
+    import atomserve_amd.models.dozusun  # noqa: F401
     import atomserve_amd.models.qwen3  # noqa: F401

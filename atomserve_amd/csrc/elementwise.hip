@@ -527,3 +527,167 @@ extern "C" int as_silu_mul(const void* gate_up, void* out, int dtype, int num_to
   else return AS_BAD_DTYPE;
   return launch_status();
 }
+
+// ---- one sum, two norms ------------------------------------------------------------------
+// A layer whose mixer and feed-forward read the same stream through a norm each:
+//   v = x[s] + (d1[s] + d2[s])        fp32; written back to x[s] if update_x (either d may be absent)
+//   out1[r] = v / sqrt(mean(v^2) + eps) * w1;   out2[r] = the same with w2 (absent: one output)
+// with s = rows ? rows[r] : r.  The root mean square is computed once.
+template <typename O, typename W>
+__global__ void rmsnorm_multi_kernel(float* __restrict__ x, const O* __restrict__ d1, const O* __restrict__ d2,
+                                     const int* __restrict__ rows, const W* __restrict__ w1,
+                                     const W* __restrict__ w2, float eps, O* __restrict__ out1,
+                                     O* __restrict__ out2, int n, int update_x) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const size_t s = rows ? (size_t)rows[r] : (size_t)r;
+  float* xr = x + s * n;
+  const O* a = d1 ? d1 + s * n : nullptr;
+  const O* b = d2 ? d2 + s * n : nullptr;
+  const bool pending = a || b;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = xr[i];
+    if (pending) {
+      v += (a ? to_f32(a[i]) : 0.f) + (b ? to_f32(b[i]) : 0.f);
+      if (update_x) xr[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = xr[i];
+    if (pending && !update_x) v += (a ? to_f32(a[i]) : 0.f) + (b ? to_f32(b[i]) : 0.f);
+    const float u = v * inv;
+    out1[(size_t)r * n + i] = from_f32<O>(u * to_f32(w1[i]));
+    if (out2) out2[(size_t)r * n + i] = from_f32<O>(u * to_f32(w2[i]));
+  }
+}
+
+extern "C" int as_rmsnorm_multi(float* x, const void* d1, const void* d2, const int* rows, const void* w1,
+                                const void* w2, int w_dtype, float eps, void* out1, void* out2, int out_dtype,
+                                int num_out_rows, int n, int update_x, hipStream_t stream) {
+  if (num_out_rows <= 0) return AS_OK;
+  if (n <= 0 || !out1 || !w1 || (out2 && !w2)) return AS_BAD_SHAPE;
+  const int threads = n >= 2048 ? 256 : (n >= 512 ? 128 : 64);
+#define LAUNCH(O, W)                                                                                        \
+  rmsnorm_multi_kernel<O, W><<<num_out_rows, threads, 0, stream>>>(x, (const O*)d1, (const O*)d2, rows,     \
+                                                                   (const W*)w1, (const W*)w2, eps, (O*)out1, \
+                                                                   (O*)out2, n, update_x)
+  if (out_dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
+  else if (out_dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
+  else if (out_dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
+  else return AS_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}
+
+// ---- heads out of a wider projection: per-head norm, padding, cache store ------------------
+// proj [T, ld] holds, among other columns, H query heads and KV key heads of `dim` coordinates and KV
+// value heads of `vdim`, starting at columns q_off, k_off, v_off.  Queries and keys are normed per head
+// (x / sqrt(mean(x^2) + eps) * weight over dim; no weights: left as they are); nothing is rotated.
+// The attention kernels take one head width for keys and values, so every head is laid out with
+// Dp >= max(dim, vdim) coordinates, the ones a head does not have being zero: scores and outputs are
+// unchanged.  q_out [T, H, Dp]; keys to k_pages [pages, KV, bs, Dp] and values transposed to v_pages
+// [pages, KV, Dp, bs] at slots[t] (page * bs + offset; negative or store == 0: not stored).
+template <typename T, typename W>
+__global__ __launch_bounds__(64) void head_norm_store_kernel(const T* __restrict__ proj, int ld, int q_off, int k_off,
+                                                             int v_off, int H, int KV, int dim, int vdim, int Dp,
+                                                             const W* __restrict__ qw, const W* __restrict__ kw,
+                                                             float eps, const int* __restrict__ slots,
+                                                             T* __restrict__ q_out, T* __restrict__ k_pages,
+                                                             T* __restrict__ v_pages, int bs, int store) {
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const T* row = proj + (size_t)t * ld;
+  if (head < H + KV) {  // a query or a key head
+    const bool is_q = head < H;
+    const int hh = is_q ? head : head - H;
+    const T* src = row + (is_q ? q_off : k_off) + hh * dim;
+    const W* w = is_q ? qw : kw;
+    T* dst;
+    if (is_q) {
+      dst = q_out + ((size_t)t * H + hh) * Dp;
+    } else {
+      const int slot = (store && slots) ? slots[t] : -1;
+      if (slot < 0) return;
+      dst = k_pages + (((size_t)(slot / bs) * KV + hh) * bs + slot % bs) * Dp;
+    }
+    float inv = 1.f;
+    if (w) {
+      float ss = 0.f;
+      for (int d = lane; d < dim; d += WAVE) { const float v = to_f32(src[d]); ss += v * v; }
+      ss = wave_sum(ss);
+      inv = 1.0f / sqrtf(ss / (float)dim + eps);
+    }
+    for (int d = lane; d < Dp; d += WAVE) {
+      float v = 0.f;
+      if (d < dim) v = w ? to_f32(src[d]) * inv * to_f32(w[d]) : to_f32(src[d]);
+      dst[d] = from_f32<T>(finite_or_zero(v));
+    }
+    return;
+  }
+  const int g = head - H - KV;  // a value head
+  const int slot = (store && slots) ? slots[t] : -1;
+  if (slot < 0) return;
+  const T* src = row + v_off + g * vdim;
+  T* dst = v_pages + ((size_t)(slot / bs) * KV + g) * Dp * bs + slot % bs;
+  for (int d = lane; d < Dp; d += WAVE) dst[(size_t)d * bs] = d < vdim ? finite_or_zero(src[d]) : from_f32<T>(0.f);
+}
+
+extern "C" int as_head_norm_store(const void* proj, int dtype, int ld, int q_off, int k_off, int v_off, int H, int KV,
+                                  int dim, int vdim, int Dp, const void* qw, const void* kw, int w_dtype, float eps,
+                                  const int* slots, void* q_out, void* k_pages, void* v_pages, int bs, int store,
+                                  int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (H <= 0 || KV <= 0 || dim <= 0 || vdim <= 0 || Dp < dim || Dp < vdim || bs <= 0 || ld <= 0 || (!qw) != (!kw))
+    return AS_BAD_SHAPE;
+  if (H + 2 * KV > 65535) return AS_BAD_SHAPE;
+  dim3 grid(num_tokens, H + 2 * KV);
+#define LAUNCH(T, W)                                                                                          \
+  head_norm_store_kernel<T, W><<<grid, 64, 0, stream>>>((const T*)proj, ld, q_off, k_off, v_off, H, KV, dim,  \
+                                                        vdim, Dp, (const W*)qw, (const W*)kw, eps, slots,     \
+                                                        (T*)q_out, (T*)k_pages, (T*)v_pages, bs, store)
+  if (dtype == DT_F32 && (w_dtype == DT_F32 || !qw)) LAUNCH(float, float);
+  else if (dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
+  else if (dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
+  else return AS_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}
+
+// ---- an output gate on attention heads --------------------------------------------------------
+// out[t, out_off + h * vdim + j] = scale * sigmoid(gate[t, gate_off + h * vdim + j]) * heads[t, h, j]
+// for j < vdim of the Dp coordinates a head is laid out with; gate [T, ld_gate], out [T, ld_out].
+template <typename T>
+__global__ void sigmoid_gate_heads_kernel(const T* __restrict__ heads, int H, int vdim, int Dp,
+                                          const T* __restrict__ gate, int ld_gate, int gate_off, float scale,
+                                          T* __restrict__ out, int ld_out, int out_off, size_t total) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const int per = H * vdim;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    const size_t t = idx / per;
+    const int c = (int)(idx % per), h = c / vdim, j = c % vdim;
+    const float g = to_f32(gate[t * ld_gate + gate_off + c]);
+    const float v = to_f32(heads[(t * H + h) * Dp + j]);
+    out[t * ld_out + out_off + c] = from_f32<T>(scale * v / (1.0f + expf(-g)));
+  }
+}
+
+extern "C" int as_sigmoid_gate_heads(const void* heads, int dtype, int H, int vdim, int Dp, const void* gate,
+                                     int ld_gate, int gate_off, float scale, void* out, int ld_out, int out_off,
+                                     int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (H <= 0 || vdim <= 0 || Dp < vdim) return AS_BAD_SHAPE;
+  const size_t total = (size_t)num_tokens * H * vdim;
+  const size_t want = (total + 255) / 256;
+  const int blocks = (int)(want > 8192 ? 8192 : want);
+  if (dtype == DT_F32)
+    sigmoid_gate_heads_kernel<float><<<blocks, 256, 0, stream>>>((const float*)heads, H, vdim, Dp, (const float*)gate,
+                                                                 ld_gate, gate_off, scale, (float*)out, ld_out, out_off, total);
+  else if (dtype == DT_BF16)
+    sigmoid_gate_heads_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)heads, H, vdim, Dp, (const bf16*)gate,
+                                                                ld_gate, gate_off, scale, (bf16*)out, ld_out, out_off, total);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}

@@ -1,0 +1,230 @@
+// Feed-forward layers made of several small experts, of which every token uses a few.
+//
+// Which experts a token uses is decided on the GPU (a table indexed by the token id here), so a step
+// never waits for the host and can be replayed as a graph.  A (token, chosen expert) is a "pair":
+// pair p = token * top + choice.  `moe_route` sorts the pairs by expert and cuts every expert's run
+// into tiles of 16; the two grouped products then take one workgroup per (tile, 64 outputs): the first
+// applies act(gate) * up on the way out, the second writes every pair's output where the pair stands
+// (so the outputs of a token's experts lie side by side), and `moe_combine` adds them up with their
+// weights.  A pair's result does not depend on what else is in the step: every output is a dot product
+// over the whole width in a fixed order.
+#include "common.h"
+
+#define MOE_TILE 16      // pairs of one expert that a workgroup takes
+#define MOE_STRIP 64     // outputs that a workgroup takes: four waves of 16
+#define MOE_MAX_EXPERTS 1024
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// ---- routing ------------------------------------------------------------------------------------
+// table [vocab, top] int32: the experts of every token id.  order [P]: the pairs sorted by expert;
+// tiles [max_tiles, 3]: (expert, first place in `order`, count <= 16); counts[0] = number of tiles.
+// One workgroup; the order of pairs within an expert is whatever the atomics make it, which no
+// result depends on.
+__global__ __launch_bounds__(1024) void moe_route_table_kernel(const int* __restrict__ token_ids,
+                                                               const int* __restrict__ table, int vocab, int top,
+                                                               int experts, int num_tokens, int* __restrict__ order,
+                                                               int* __restrict__ tiles, int* __restrict__ counts,
+                                                               int max_tiles) {
+  __shared__ int hist[MOE_MAX_EXPERTS];
+  __shared__ int cursor[MOE_MAX_EXPERTS];
+  const int P = num_tokens * top;
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) hist[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    int id = token_ids[p / top];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    int e = table[(size_t)id * top + p % top];
+    e = e < 0 ? 0 : (e >= experts ? experts - 1 : e);
+    atomicAdd(&hist[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, n = 0;
+    for (int e = 0; e < experts; ++e) {
+      cursor[e] = at;
+      for (int s = 0; s < hist[e] && n < max_tiles; s += MOE_TILE, ++n) {
+        tiles[3 * n] = e;
+        tiles[3 * n + 1] = at + s;
+        tiles[3 * n + 2] = min(MOE_TILE, hist[e] - s);
+      }
+      at += hist[e];
+    }
+    counts[0] = n;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    int id = token_ids[p / top];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    int e = table[(size_t)id * top + p % top];
+    e = e < 0 ? 0 : (e >= experts ? experts - 1 : e);
+    order[atomicAdd(&cursor[e], 1)] = p;
+  }
+}
+
+extern "C" int as_moe_route_table(const int* token_ids, const int* table, int vocab, int top, int experts,
+                                  int num_tokens, int* order, int* tiles, int* counts, int max_tiles,
+                                  hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (top <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || vocab <= 0) return AS_BAD_SHAPE;
+  if (max_tiles < (num_tokens * top + MOE_TILE - 1) / MOE_TILE + experts) return AS_BAD_SHAPE;
+  moe_route_table_kernel<<<1, 1024, 0, stream>>>(token_ids, table, vocab, top, experts, num_tokens, order, tiles,
+                                                 counts, max_tiles);
+  return launch_status();
+}
+
+// ---- the grouped products -------------------------------------------------------------------------
+// a: the inputs, a row per token (pair p reads row p / a_div: a_div = top for the first product, 1 for
+// the second, whose inputs are the first one's outputs, a row per pair).  w [experts, N_w, K].
+// GATED: N_w = 2 N, rows 0..N-1 the gate, N..2N-1 the up projection; out[p, n] = silu(gate) * up.
+// else:  out[p, n] = the product.  out has a row per pair.
+//
+// bf16: v_mfma_f32_16x16x32_bf16 with the weights as the A operand (16 rows of w) and the tile's 16
+// pairs as the B operand; a wave owns 16 outputs (and their up rows), walks K in steps of 32 and reads
+// both operands straight from memory, 16 bytes a lane.  Needs K % 8 == 0.
+template <bool GATED, typename OutT>
+__global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restrict__ a, int a_div,
+                                                            const bf16* __restrict__ w, int N, int K,
+                                                            const int* __restrict__ order,
+                                                            const int* __restrict__ tiles,
+                                                            const int* __restrict__ counts, OutT* __restrict__ out) {
+  const int tile = blockIdx.y;
+  if (tile >= counts[0]) return;
+  const int e = tiles[3 * tile], at = tiles[3 * tile + 1], cnt = tiles[3 * tile + 2];
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int n0 = blockIdx.x * MOE_STRIP + wave * 16;
+  if (n0 >= N) return;
+  const int pair = lr < cnt ? order[at + lr] : -1;  // this lane's column of the B operand
+  const bf16* arow = pair >= 0 ? a + (size_t)(pair / a_div) * K : nullptr;
+  const int NW = GATED ? 2 * N : N;
+  const bf16* wbase = w + (size_t)e * NW * K;
+  const bool row_in = n0 + lr < N;
+  const bf16* wrow = wbase + (size_t)(n0 + lr) * K;
+  const bf16* urow = wbase + (size_t)(N + n0 + lr) * K;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f}, acc_up = {0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const int k = k0 + lg * 8;
+    const bool k_in = k < K;
+    const bf16x8 av = (arow && k_in) ? *reinterpret_cast<const bf16x8*>(arow + k) : zero;
+    const bf16x8 wv = (row_in && k_in) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc, 0, 0, 0);
+    if (GATED) {
+      const bf16x8 uv = (row_in && k_in) ? *reinterpret_cast<const bf16x8*>(urow + k) : zero;
+      acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv, av, acc_up, 0, 0, 0);
+    }
+  }
+  // a lane holds outputs n0 + 4 lg + i (i < 4) of the pair in column lr
+  if (pair < 0) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = n0 + 4 * lg + i;
+    if (n >= N) continue;
+    float v = acc[i];
+    if (GATED) {
+      const float g = to_f32((bf16)acc[i]), u = to_f32((bf16)acc_up[i]);  // the two products rounded as if stored
+      v = g / (1.0f + expf(-g)) * u;
+    }
+    out[(size_t)pair * N + n] = from_f32<OutT>(v);
+  }
+}
+
+// fp32: plain multiply-add, every output one chain over k in order.  A thread owns an output and four
+// of the tile's sixteen pairs.
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_gemm_f32_kernel(const float* __restrict__ a, int a_div,
+                                                           const float* __restrict__ w, int N, int K,
+                                                           const int* __restrict__ order,
+                                                           const int* __restrict__ tiles,
+                                                           const int* __restrict__ counts, float* __restrict__ out) {
+  const int tile = blockIdx.y;
+  if (tile >= counts[0]) return;
+  const int e = tiles[3 * tile], at = tiles[3 * tile + 1], cnt = tiles[3 * tile + 2];
+  const int n = blockIdx.x * MOE_STRIP + (threadIdx.x & 63), quarter = threadIdx.x >> 6;
+  if (n >= N) return;
+  const int NW = GATED ? 2 * N : N;
+  const float* wrow = w + ((size_t)e * NW + n) * K;
+  const float* urow = w + ((size_t)e * NW + N + n) * K;
+  int pairs[4];
+  const float* arow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int place = quarter * 4 + i;
+    pairs[i] = place < cnt ? order[at + place] : -1;
+    arow[i] = a + (size_t)(pairs[i] < 0 ? 0 : pairs[i] / a_div) * K;
+  }
+  float acc[4] = {0.f, 0.f, 0.f, 0.f}, acc_up[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k = 0; k < K; ++k) {
+    const float wv = wrow[k], uv = GATED ? urow[k] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float av = arow[i][k];
+      acc[i] = fmaf(wv, av, acc[i]);
+      if (GATED) acc_up[i] = fmaf(uv, av, acc_up[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (pairs[i] < 0) continue;
+    float v = acc[i];
+    if (GATED) v = v / (1.0f + expf(-v)) * acc_up[i];
+    out[(size_t)pairs[i] * N + n] = v;
+  }
+}
+
+// out_dtype: DT_BF16 or DT_F32 for the bf16 product's results (fp32 where several experts' outputs
+// are still to be added up); the fp32 product writes fp32.
+extern "C" int as_moe_gemm(const void* a, int dtype, int a_div, const void* w, int N, int K, int gated, const int* order,
+                           const int* tiles, const int* counts, int max_tiles, void* out, int out_dtype,
+                           hipStream_t stream) {
+  if (max_tiles <= 0) return AS_OK;
+  if (N <= 0 || K <= 0 || a_div <= 0 || max_tiles > 65535) return AS_BAD_SHAPE;
+  dim3 grid((N + MOE_STRIP - 1) / MOE_STRIP, max_tiles);
+  if (dtype == DT_F32) {
+    if (out_dtype != DT_F32) return AS_BAD_DTYPE;
+    if (gated) moe_gemm_f32_kernel<true><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out);
+    else moe_gemm_f32_kernel<false><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out);
+    return launch_status();
+  }
+  if (dtype != DT_BF16) return AS_BAD_DTYPE;
+  if (K & 7) return AS_BAD_SHAPE;
+  if (gated) {
+    if (out_dtype != DT_BF16) return AS_BAD_DTYPE;
+    moe_gemm_bf16_kernel<true, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out);
+  } else if (out_dtype == DT_BF16) {
+    moe_gemm_bf16_kernel<false, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out);
+  } else if (out_dtype == DT_F32) {
+    moe_gemm_bf16_kernel<false, float><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (float*)out);
+  } else {
+    return AS_BAD_DTYPE;
+  }
+  return launch_status();
+}
+
+// out[t, n] = sum over a token's `top` pairs of weight * pair_out[t * top + j, n]  (fp32 in, T out).
+template <typename T>
+__global__ void moe_combine_kernel(const float* __restrict__ pair_out, int top, float weight, int N,
+                                   T* __restrict__ out, size_t total) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    const size_t t = idx / N;
+    const int n = (int)(idx % N);
+    float s = 0.f;
+    for (int j = 0; j < top; ++j) s += weight * pair_out[(t * top + j) * N + n];
+    out[idx] = from_f32<T>(s);
+  }
+}
+
+extern "C" int as_moe_combine(const float* pair_out, int top, float weight, int N, void* out, int out_dtype,
+                              int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (top <= 0 || N <= 0) return AS_BAD_SHAPE;
+  const size_t total = (size_t)num_tokens * N, want = (total + 255) / 256;
+  const int blocks = (int)(want > 8192 ? 8192 : want);
+  if (out_dtype == DT_F32) moe_combine_kernel<float><<<blocks, 256, 0, stream>>>(pair_out, top, weight, N, (float*)out, total);
+  else if (out_dtype == DT_BF16) moe_combine_kernel<bf16><<<blocks, 256, 0, stream>>>(pair_out, top, weight, N, (bf16*)out, total);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}

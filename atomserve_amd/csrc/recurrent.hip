@@ -1,0 +1,425 @@
+// Mixers that carry a fixed-size state from token to token: short causal convolutions, the gated
+// delta rule and the gated linear recurrence.  Everything that enters a recurrence (decays, step
+// sizes, gates, unit norms, the state itself) is fp32 in both precisions; only what the matrix
+// products hand over (T) and the activations handed on to the next product are bf16 when serving.
+//
+// A step's rows are described as everywhere else: tok_row [T] (the row of a token), and per row its
+// first flat token, its length, the position of its first token and its slot in the state tables.  A
+// row that starts at position 0 starts from a zero state whatever its slot holds (slots are used
+// again); a portion of a prompt goes on from what the portion before left.  State tables are fp32
+// [slots, ...]; a row's state is written back only when `writes`.
+#include "common.h"
+
+#define CONV_MAX_TAPS 8
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+__device__ __forceinline__ float siluf_(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float gelu_tanhf_(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// ---- short causal convolution per channel ------------------------------------------------------
+// in [T, ld]: the C channels start at column col0; in_bias [C] (or none) is added to every input that
+// exists (the zeros before a sequence stay zeros).  w [C, taps], the last column multiplying the
+// current token; bias [C] or none; act 1: silu.  history [slots, taps - 1, C]: the inputs of the last
+// taps - 1 tokens before the row, oldest first.  out fp32 [T, C].
+template <typename T, typename W>
+__global__ void short_conv_kernel(const T* __restrict__ in, int ld, int col0, int C, const W* __restrict__ in_bias,
+                                  const W* __restrict__ w, const W* __restrict__ bias, int taps, int act,
+                                  const float* __restrict__ history, const int* __restrict__ tok_row,
+                                  const int* __restrict__ row_first, const int* __restrict__ row_start,
+                                  const int* __restrict__ row_slots, float* __restrict__ out) {
+  const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int r = tok_row ? tok_row[t] : t;
+  const int first = row_first[r], j = t - first;
+  const bool carried = row_start[r] > 0 && row_slots[r] >= 0;
+  const float* old = history + (size_t)(carried ? row_slots[r] : 0) * (taps - 1) * C;
+  const float ib = in_bias ? to_f32(in_bias[c]) : 0.f;
+  float acc = 0.f;
+  for (int i = 0; i < taps; ++i) {
+    const int src = j - (taps - 1 - i);
+    float v = 0.f;
+    if (src >= 0) v = to_f32(in[(size_t)(first + src) * ld + col0 + c]) + ib;
+    else if (carried) v = old[(size_t)(taps - 1 + src) * C + c];
+    acc = fmaf(to_f32(w[(size_t)c * taps + i]), v, acc);
+  }
+  if (bias) acc += to_f32(bias[c]);
+  out[(size_t)t * C + c] = act == 1 ? siluf_(acc) : acc;
+}
+
+// After the convolution: the history of every row moves on by the row's tokens.
+template <typename T, typename W>
+__global__ void conv_history_kernel(const T* __restrict__ in, int ld, int col0, int C, const W* __restrict__ in_bias,
+                                    int taps, float* __restrict__ history, const int* __restrict__ row_first,
+                                    const int* __restrict__ row_len, const int* __restrict__ row_start,
+                                    const int* __restrict__ row_slots) {
+  const int r = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C || row_slots[r] < 0) return;
+  const int first = row_first[r], len = row_len[r], keep = taps - 1;
+  float* mine = history + (size_t)row_slots[r] * keep * C;
+  const bool carried = row_start[r] > 0;
+  const float ib = in_bias ? to_f32(in_bias[c]) : 0.f;
+  float fresh[CONV_MAX_TAPS];
+  for (int h = 0; h < keep; ++h) {
+    const int src = len - keep + h;  // among the row's tokens; negative: among the old history
+    if (src >= 0) fresh[h] = to_f32(in[(size_t)(first + src) * ld + col0 + c]) + ib;
+    else fresh[h] = carried ? mine[(size_t)(keep + src) * C + c] : 0.f;
+  }
+  for (int h = 0; h < keep; ++h) mine[(size_t)h * C + c] = fresh[h];
+}
+
+extern "C" int as_short_conv(const void* in, int dtype, int ld, int col0, int C, const void* in_bias, const void* w,
+                             const void* bias, int w_dtype, int taps, int act, float* history, const int* tok_row,
+                             const int* row_first, const int* row_len, const int* row_start, const int* row_slots,
+                             float* out, int num_tokens, int num_rows, int writes, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (C <= 0 || taps < 1 || taps > CONV_MAX_TAPS || ld < col0 + C || num_rows <= 0) return AS_BAD_SHAPE;
+  const int threads = C >= 256 ? 256 : 64;
+  dim3 grid(num_tokens, (C + threads - 1) / threads), rows_grid(num_rows, (C + threads - 1) / threads);
+  if (grid.y > 65535) return AS_BAD_SHAPE;
+#define LAUNCH(T, W)                                                                                              \
+  do {                                                                                                            \
+    short_conv_kernel<T, W><<<grid, threads, 0, stream>>>((const T*)in, ld, col0, C, (const W*)in_bias,          \
+                                                          (const W*)w, (const W*)bias, taps, act, history,       \
+                                                          tok_row, row_first, row_start, row_slots, out);        \
+    if (writes && taps > 1)                                                                                       \
+      conv_history_kernel<T, W><<<rows_grid, threads, 0, stream>>>((const T*)in, ld, col0, C, (const W*)in_bias, \
+                                                                   taps, history, row_first, row_len, row_start, \
+                                                                   row_slots);                                    \
+  } while (0)
+  if (dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
+  else if (dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
+  else if (dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
+  else return AS_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}
+
+// ---- gated delta rule ----------------------------------------------------------------------------
+// Before the scan, per token: the query and key heads (G of them, `dim` wide, in qkv [T, C] at columns
+// 0 and G * dim) become unit vectors, x / sqrt(sum(x^2) + 1e-6), the query also times dim^(-1/2); per
+// value head beta = sigmoid(b) and the decay g = exp(-exp(A_log) * softplus(a + dt_bias)), with b and a
+// taken from the projection's output proj [T, ld] at columns b_off and a_off.
+template <typename T, typename W>
+__global__ __launch_bounds__(256) void delta_prepare_kernel(float* __restrict__ qkv, int C, int G, int dim, int H,
+                                                            const T* __restrict__ proj, int ld, int b_off, int a_off,
+                                                            const W* __restrict__ a_log, const W* __restrict__ dt_bias,
+                                                            float* __restrict__ beta, float* __restrict__ decay) {
+  const int t = blockIdx.x, lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
+  float* row = qkv + (size_t)t * C;
+  for (int head = wave; head < 2 * G; head += waves) {
+    float* x = row + (size_t)head * dim;  // query heads first, then key heads
+    float ss = 0.f;
+    for (int d = lane; d < dim; d += WAVE) ss += x[d] * x[d];
+    ss = wave_sum(ss);
+    float f = 1.0f / sqrtf(ss + 1e-6f);
+    if (head < G) f *= 1.0f / sqrtf((float)dim);
+    for (int d = lane; d < dim; d += WAVE) x[d] *= f;
+  }
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    const float b = to_f32(proj[(size_t)t * ld + b_off + h]), a = to_f32(proj[(size_t)t * ld + a_off + h]);
+    beta[(size_t)t * H + h] = sigmoidf_(b);
+    decay[(size_t)t * H + h] = expf(-expf(to_f32(a_log[h])) * softplusf_(a + to_f32(dt_bias[h])));
+  }
+}
+
+extern "C" int as_delta_prepare(float* qkv, int C, int G, int dim, int H, const void* proj, int dtype, int ld, int b_off,
+                                int a_off, const void* a_log, const void* dt_bias, int w_dtype, float* beta,
+                                float* decay, int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (G <= 0 || dim <= 0 || H <= 0 || C < 2 * G * dim) return AS_BAD_SHAPE;
+#define LAUNCH(T, W)                                                                                               \
+  delta_prepare_kernel<T, W><<<num_tokens, 256, 0, stream>>>(qkv, C, G, dim, H, (const T*)proj, ld, b_off, a_off,  \
+                                                             (const W*)a_log, (const W*)dt_bias, beta, decay)
+  if (dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
+  else if (dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
+  else if (dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
+  else return AS_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}
+
+// The scan.  Per head the state S [dim, vdim] moves on token by token:
+//   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q     (o sees the token's own write)
+// The columns of S never meet, so a wave owns CJ columns of one head of one row and keeps them in
+// registers for all the row's tokens: lane = slice * CJ + column, a slice being RPL rows of S
+// (64 / CJ slices cover dim).  With p = S_old^T k and r = S_old^T q, both taken in one pass over the
+// old state:  u = beta (v - g p),  S_new = g S_old + k u^T,  o = g r + u (k . q).
+// Keys and queries of TB tokens at a time go through LDS (one round of loads per TB tokens, not one
+// per token).
+#define DELTA_TB 8
+template <int RPL>
+__global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ qkv, int C, int G, int dim, int H,
+                                                        int vdim, int CJ, const float* __restrict__ beta,
+                                                        const float* __restrict__ decay, float* __restrict__ state,
+                                                        const int* __restrict__ row_first,
+                                                        const int* __restrict__ row_len,
+                                                        const int* __restrict__ row_start,
+                                                        const int* __restrict__ row_slots, int writes,
+                                                        float* __restrict__ out) {
+  extern __shared__ float lds[];  // [DELTA_TB][2][dimp]: key then query of each token, dimp = slices * RPL
+  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int col = lane % CJ, slice = lane / CJ, slices = WAVE / CJ;
+  const int dimp = slices * RPL;
+  const int j = blockIdx.z * CJ + col;
+  const bool live = j < vdim;
+  const int g = h / (H / G);
+  const int first = row_first[r], len = row_len[r], slot = row_slots[r];
+  const int i0 = slice * RPL;
+  float S[RPL];
+  float* mine = state + ((size_t)(slot < 0 ? 0 : slot) * H + h) * dim * vdim;
+  const bool carried = row_start[r] > 0 && slot >= 0;
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) S[i] = (carried && live && i0 + i < dim) ? mine[(size_t)(i0 + i) * vdim + j] : 0.f;
+  const int q_col = g * dim, k_col = (G + g) * dim, v_col = 2 * G * dim + h * vdim;
+  for (int t0 = 0; t0 < len; t0 += DELTA_TB) {
+    const int nt = min(DELTA_TB, len - t0);
+    __syncthreads();
+    for (int e = lane; e < nt * 2 * dimp; e += WAVE) {
+      const int tt = e / (2 * dimp), rest = e % (2 * dimp), which = rest / dimp, i = rest % dimp;
+      lds[e] = i < dim ? qkv[(size_t)(first + t0 + tt) * C + (which ? q_col : k_col) + i] : 0.f;
+    }
+    float vj[DELTA_TB], bt[DELTA_TB], gt[DELTA_TB];
+#pragma unroll
+    for (int tt = 0; tt < DELTA_TB; ++tt) {
+      const size_t t = (size_t)first + t0 + (tt < nt ? tt : 0);
+      vj[tt] = live ? qkv[t * C + v_col + j] : 0.f;
+      bt[tt] = beta[t * H + h];
+      gt[tt] = decay[t * H + h];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < DELTA_TB; ++tt) {
+      if (tt < nt) {
+        const float* kk = lds + (size_t)tt * 2 * dimp + i0;
+        const float* qq = kk + dimp;
+        float p = 0.f, rr = 0.f, kq = 0.f;
+#pragma unroll
+        for (int i = 0; i < RPL; ++i) {
+          p = fmaf(S[i], kk[i], p);
+          rr = fmaf(S[i], qq[i], rr);
+          kq = fmaf(kk[i], qq[i], kq);
+        }
+        for (int off = CJ; off < WAVE; off <<= 1) {
+          p += __shfl_xor(p, off, WAVE);
+          rr += __shfl_xor(rr, off, WAVE);
+          kq += __shfl_xor(kq, off, WAVE);
+        }
+        const float gg = gt[tt];
+        const float u = bt[tt] * (vj[tt] - gg * p);
+#pragma unroll
+        for (int i = 0; i < RPL; ++i) S[i] = fmaf(kk[i], u, gg * S[i]);
+        if (live && slice == 0) out[((size_t)(first + t0 + tt) * H + h) * vdim + j] = fmaf(gg, rr, u * kq);
+      }
+    }
+  }
+  if (writes && live && slot >= 0) {
+#pragma unroll
+    for (int i = 0; i < RPL; ++i)
+      if (i0 + i < dim) mine[(size_t)(i0 + i) * vdim + j] = S[i];
+  }
+}
+
+extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int vdim, const float* beta,
+                             const float* decay, float* state, const int* row_first, const int* row_len,
+                             const int* row_start, const int* row_slots, int writes, float* out, int num_rows,
+                             hipStream_t stream) {
+  if (num_rows <= 0) return AS_OK;
+  if (G <= 0 || H <= 0 || H % G || dim <= 0 || vdim <= 0 || dim > 64 * 64 || C < 2 * G * dim + H * vdim || H > 65535)
+    return AS_BAD_SHAPE;
+  int slices = 1;
+  while ((dim + slices - 1) / slices > 64) slices *= 2;  // a lane keeps at most 64 rows of its column
+  const int rows_per_lane = (dim + slices - 1) / slices;
+  const int RPL = rows_per_lane <= 8 ? 8 : rows_per_lane <= 16 ? 16 : rows_per_lane <= 32 ? 32 : 64;
+  const int CJ = WAVE / slices;
+  dim3 grid(num_rows, H, (vdim + CJ - 1) / CJ);
+  const size_t lds = (size_t)DELTA_TB * 2 * slices * RPL * sizeof(float);
+#define LAUNCH(R)                                                                                              \
+  delta_scan_kernel<R><<<grid, 64, lds, stream>>>(qkv, C, G, dim, H, vdim, CJ, beta, decay, state, row_first,  \
+                                                  row_len, row_start, row_slots, writes, out)
+  if (RPL == 8) LAUNCH(8);
+  else if (RPL == 16) LAUNCH(16);
+  else if (RPL == 32) LAUNCH(32);
+  else LAUNCH(64);
+#undef LAUNCH
+  return launch_status();
+}
+
+// After the scan: every head's output over its root mean square (over vdim, eps inside the root), times
+// a weight [vdim] shared by the heads, times silu of the gate projection's output (proj [T, ld] at
+// g_off, laid out heads x vdim): the input of the output projection, [T, H * vdim] in T.
+template <typename T, typename W>
+__global__ __launch_bounds__(64) void delta_finish_kernel(const float* __restrict__ o, int H, int vdim,
+                                                          const W* __restrict__ w, float eps,
+                                                          const T* __restrict__ proj, int ld, int g_off,
+                                                          T* __restrict__ act) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* x = o + ((size_t)t * H + h) * vdim;
+  float ss = 0.f;
+  for (int d = lane; d < vdim; d += WAVE) ss += x[d] * x[d];
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+  for (int d = lane; d < vdim; d += WAVE) {
+    const float gate = to_f32(proj[(size_t)t * ld + g_off + h * vdim + d]);
+    act[((size_t)t * H + h) * vdim + d] = from_f32<T>(x[d] * inv * to_f32(w[d]) * siluf_(gate));
+  }
+}
+
+extern "C" int as_delta_finish(const float* o, int H, int vdim, const void* w, int w_dtype, float eps, const void* proj,
+                               int dtype, int ld, int g_off, void* act, int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (H <= 0 || H > 65535 || vdim <= 0) return AS_BAD_SHAPE;
+  dim3 grid(num_tokens, H);
+#define LAUNCH(T, W)                                                                                             \
+  delta_finish_kernel<T, W><<<grid, 64, 0, stream>>>(o, H, vdim, (const W*)w, eps, (const T*)proj, ld, g_off, (T*)act)
+  if (dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
+  else if (dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
+  else if (dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
+  else return AS_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}
+
+// ---- gated linear recurrence ----------------------------------------------------------------------
+// The gates.  u fp32 [T, width] is cut into `blocks` parts of bw channels; in part b
+//   r = sigmoid(ra[b] u_b + ra_b[b]),  i = sigmoid(ri[b] u_b + ri_b[b])     (ra, ri [blocks, bw, bw], out x in)
+//   a = exp(-c r softplus(lam));  a_out = a,  x_out = sqrt(1 - a^2) i u.
+// A workgroup takes 32 tokens by 64 outputs of one part; tokens and weights meet in LDS in pieces of
+// 32 inputs; every output is one fma chain over its inputs in order, whatever shares the launch.
+#define GATE_TT 32
+#define GATE_TO 64
+#define GATE_KC 32
+template <typename W>
+__global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restrict__ u, int width, int bw,
+                                                          const W* __restrict__ ra, const W* __restrict__ ra_b,
+                                                          const W* __restrict__ ri, const W* __restrict__ ri_b,
+                                                          const W* __restrict__ lam, float c, float* __restrict__ a_out,
+                                                          float* __restrict__ x_out, int num_tokens) {
+  __shared__ float us[GATE_TT][GATE_KC + 1];
+  __shared__ float wr[GATE_TO][GATE_KC + 1];
+  __shared__ float wi[GATE_TO][GATE_KC + 1];
+  const int b = blockIdx.y, t0 = blockIdx.x * GATE_TT, o0 = blockIdx.z * GATE_TO;
+  const int tx = threadIdx.x % GATE_TO, ty = threadIdx.x / GATE_TO;  // an output, and 8 of the 32 tokens
+  float accr[8] = {}, acci[8] = {};
+  const W* rab = ra + (size_t)b * bw * bw;
+  const W* rib = ri + (size_t)b * bw * bw;
+  for (int k0 = 0; k0 < bw; k0 += GATE_KC) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < GATE_TT * GATE_KC; e += 256) {
+      const int tt = e / GATE_KC, kk = e % GATE_KC;
+      us[tt][kk] = (t0 + tt < num_tokens && k0 + kk < bw) ? u[(size_t)(t0 + tt) * width + b * bw + k0 + kk] : 0.f;
+    }
+    for (int e = threadIdx.x; e < GATE_TO * GATE_KC; e += 256) {
+      const int oo = e / GATE_KC, kk = e % GATE_KC;
+      const bool in = o0 + oo < bw && k0 + kk < bw;
+      wr[oo][kk] = in ? to_f32(rab[(size_t)(o0 + oo) * bw + k0 + kk]) : 0.f;
+      wi[oo][kk] = in ? to_f32(rib[(size_t)(o0 + oo) * bw + k0 + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < GATE_KC; ++kk) {
+      const float a = wr[tx][kk], bb = wi[tx][kk];
+#pragma unroll
+      for (int tt = 0; tt < 8; ++tt) {
+        const float uu = us[ty * 8 + tt][kk];
+        accr[tt] = fmaf(a, uu, accr[tt]);
+        acci[tt] = fmaf(bb, uu, acci[tt]);
+      }
+    }
+  }
+  const int o = o0 + tx;
+  if (o >= bw) return;
+  const int ch = b * bw + o;
+  const float rb = to_f32(ra_b[ch]), ib = to_f32(ri_b[ch]), sp = softplusf_(to_f32(lam[ch]));
+#pragma unroll
+  for (int tt = 0; tt < 8; ++tt) {
+    const int t = t0 + ty * 8 + tt;
+    if (t >= num_tokens) continue;
+    const float rg = sigmoidf_(accr[tt] + rb), ig = sigmoidf_(acci[tt] + ib);
+    const float log_a = -c * rg * sp;
+    a_out[(size_t)t * width + ch] = expf(log_a);
+    x_out[(size_t)t * width + ch] = sqrtf(-expm1f(2.0f * log_a)) * ig * u[(size_t)t * width + ch];
+  }
+}
+
+extern "C" int as_rglru_gates(const float* u, int width, int blocks, const void* ra, const void* ra_b, const void* ri,
+                              const void* ri_b, const void* lam, int w_dtype, float c, float* a_out, float* x_out,
+                              int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (width <= 0 || blocks <= 0 || width % blocks || blocks > 65535) return AS_BAD_SHAPE;
+  const int bw = width / blocks;
+  dim3 grid((num_tokens + GATE_TT - 1) / GATE_TT, blocks, (bw + GATE_TO - 1) / GATE_TO);
+  if (grid.z > 65535) return AS_BAD_SHAPE;
+  if (w_dtype == DT_F32)
+    rglru_gates_kernel<float><<<grid, 256, 0, stream>>>(u, width, bw, (const float*)ra, (const float*)ra_b,
+                                                        (const float*)ri, (const float*)ri_b, (const float*)lam, c,
+                                                        a_out, x_out, num_tokens);
+  else if (w_dtype == DT_BF16)
+    rglru_gates_kernel<bf16><<<grid, 256, 0, stream>>>(u, width, bw, (const bf16*)ra, (const bf16*)ra_b,
+                                                       (const bf16*)ri, (const bf16*)ri_b, (const bf16*)lam, c, a_out,
+                                                       x_out, num_tokens);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// The scan: S = a S + x per channel, from zero at the start of a sequence; what leaves is
+// scale * S * gelu_tanh(y + y_bias) with y from proj [T, ld] at y_off, into out [T, ld_out] at out_off.
+// A thread owns a channel of a row; the loads of four tokens are asked for together.
+template <typename T, typename W>
+__global__ void rglru_scan_kernel(const float* __restrict__ a, const float* __restrict__ x, int width,
+                                  const T* __restrict__ proj, int ld, int y_off, const W* __restrict__ y_bias,
+                                  float scale, float* __restrict__ state, const int* __restrict__ row_first,
+                                  const int* __restrict__ row_len, const int* __restrict__ row_start,
+                                  const int* __restrict__ row_slots, int writes, T* __restrict__ out, int ld_out,
+                                  int out_off) {
+  const int r = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int first = row_first[r], len = row_len[r], slot = row_slots[r];
+  float* mine = state + (size_t)(slot < 0 ? 0 : slot) * width + c;
+  float S = (row_start[r] > 0 && slot >= 0) ? *mine : 0.f;
+  const float yb = y_bias ? to_f32(y_bias[c]) : 0.f;
+  int j = 0;
+  for (; j + 4 <= len; j += 4) {
+    float av[4], xv[4], yv[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const size_t t = (size_t)first + j + k;
+      av[k] = a[t * width + c];
+      xv[k] = x[t * width + c];
+      yv[k] = to_f32(proj[t * ld + y_off + c]);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      S = fmaf(av[k], S, xv[k]);
+      out[((size_t)first + j + k) * ld_out + out_off + c] = from_f32<T>(scale * S * gelu_tanhf_(yv[k] + yb));
+    }
+  }
+  for (; j < len; ++j) {
+    const size_t t = (size_t)first + j;
+    S = fmaf(a[t * width + c], S, x[t * width + c]);
+    out[t * ld_out + out_off + c] = from_f32<T>(scale * S * gelu_tanhf_(to_f32(proj[t * ld + y_off + c]) + yb));
+  }
+  if (writes && slot >= 0) *mine = S;
+}
+
+extern "C" int as_rglru_scan(const float* a, const float* x, int width, const void* proj, int dtype, int ld, int y_off,
+                             const void* y_bias, int w_dtype, float scale, float* state, const int* row_first,
+                             const int* row_len, const int* row_start, const int* row_slots, int writes, void* out,
+                             int ld_out, int out_off, int num_rows, hipStream_t stream) {
+  if (num_rows <= 0) return AS_OK;
+  if (width <= 0 || num_rows > 65535 || ld < y_off + width || ld_out < out_off + width) return AS_BAD_SHAPE;
+  const int threads = width >= 1024 ? 256 : 64;
+  dim3 grid((width + threads - 1) / threads, num_rows);
+#define LAUNCH(T, W)                                                                                              \
+  rglru_scan_kernel<T, W><<<grid, threads, 0, stream>>>(a, x, width, (const T*)proj, ld, y_off, (const W*)y_bias, \
+                                                        scale, state, row_first, row_len, row_start, row_slots,  \
+                                                        writes, (T*)out, ld_out, out_off)
+  if (dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
+  else if (dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
+  else if (dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
+  else return AS_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}

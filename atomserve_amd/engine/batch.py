@@ -349,9 +349,13 @@ class StepBatch:
         return True
 
     def cache_view(self, cache_id: int, writes: bool):
-        """The view of cache `cache_id` for a mixer in this step; None for a mixer that keeps nothing."""
+        """The view of cache `cache_id` for a mixer in this step; None for a mixer that keeps nothing; a dict
+        name -> view for a mixer that keeps several things."""
         found = self.pools.manager.group_of_cache.get(cache_id)
         if found is None:
+            names = self.pools.manager.names_of_cache.get(cache_id)
+            if names:
+                return {name: self.cache_view((cache_id, name), writes) for name in names}
             return None
         kind, gi, _ = found
         if kind == "paged":

@@ -997,3 +997,289 @@ def topk(logits, k, values, indices) -> None:
     _check(values, "values", F32, (B, k))
     _check(indices, "indices", I32, (B, k))
     call("as_topk", _ptr(logits), B, V, k, _ptr(values), _ptr(indices), _stream())
+
+
+# ---- layers whose parts read one stream side by side -------------------------------------------------
+
+
+def rmsnorm_multi(x, weight1, weight2, eps, out1, out2=None, delta1=None, delta2=None, rows=None, update_x=True) -> None:
+    """v = x[s] + (delta1[s] + delta2[s]) (either may be absent), s = rows[r] or r; out1[r] = norm(v) * weight1 and,
+    if given, out2[r] = norm(v) * weight2, the root mean square taken once; x fp32 [T, n] receives v when
+    `update_x` and something was added."""
+    _check(x, "x", F32, (None, None))
+    T, n = x.shape
+    n_out = T
+    if rows is not None:
+        _check(rows, "rows", I32, (None,))
+        n_out = rows.shape[0]
+    _check(out1, "out1", (F32, BF16), (n_out, n))
+    _check(weight1, "weight1", (F32, BF16), (n,))
+    if out1.dtype == F32 and weight1.dtype != F32:
+        raise KernelError("fp32 norm needs an fp32 weight")
+    if (out2 is None) != (weight2 is None):
+        raise KernelError("a second output and a second weight come together")
+    if out2 is not None:
+        _check(out2, "out2", out1.dtype, (n_out, n))
+        _check(weight2, "weight2", weight1.dtype, (n,))
+    for name, d in (("delta1", delta1), ("delta2", delta2)):
+        if d is not None:
+            _check(d, name, out1.dtype, (T, n))
+    call("as_rmsnorm_multi", _ptr(x), _ptr(delta1), _ptr(delta2), _ptr(rows), _ptr(weight1), _ptr(weight2),
+         _DT[weight1.dtype], float(eps), _ptr(out1), _ptr(out2), _DT[out1.dtype], n_out, n, int(bool(update_x)), _stream())  # fmt: skip
+
+
+def head_norm_store(proj, q_off, k_off, v_off, num_heads, num_kv_heads, dim, vdim, q_weight, k_weight, eps, slots,
+                    q_out, k_pages, v_pages, store_kv=True) -> None:  # fmt: skip
+    """Heads cut out of a wider projection's output proj [T, ld] (queries at column q_off, keys at k_off, both
+    `dim` wide; values at v_off, `vdim` wide): per-head RMS norm of queries and keys (weights [dim], or none), no
+    rotation, and the cache store.  Every head is laid out Dp = q_out.shape[2] >= max(dim, vdim) wide, zero where
+    it has no coordinate: q_out [T, H, Dp], k_pages [pages, KV, bs, Dp], v_pages [pages, KV, Dp, bs]."""
+    _check(proj, "proj", (F32, BF16), (None, None))
+    T, ld = proj.shape
+    H, KV = num_heads, num_kv_heads
+    _check(q_out, "q_out", proj.dtype, (T, H, None))
+    Dp = q_out.shape[2]
+    if Dp < max(dim, vdim) or min(q_off, k_off, v_off) < 0 or q_off + H * dim > ld or k_off + KV * dim > ld \
+            or v_off + KV * vdim > ld:  # fmt: skip
+        raise KernelError("head_norm_store: heads lie outside the projection's columns or the padded head width")
+    w_dtype = proj.dtype
+    if q_weight is not None:
+        _check(q_weight, "q_weight", (F32, BF16), (dim,))
+        _check(k_weight, "k_weight", q_weight.dtype, (dim,))
+        w_dtype = q_weight.dtype
+        if proj.dtype == F32 and w_dtype != F32:
+            raise KernelError("fp32 q/k norm needs fp32 weights")
+    elif k_weight is not None:
+        raise KernelError("q and k norm weights come together")
+    bs = 1
+    if store_kv:
+        _check(slots, "slots", I32, (T,))
+        _check(k_pages, "k_pages", proj.dtype, (None, KV, None, Dp))
+        bs = k_pages.shape[2]
+        _check(v_pages, "v_pages", proj.dtype, (k_pages.shape[0], KV, Dp, bs))
+    call("as_head_norm_store", _ptr(proj), _DT[proj.dtype], ld, q_off, k_off, v_off, H, KV, dim, vdim, Dp,
+         _ptr(q_weight), _ptr(k_weight), _DT[w_dtype], float(eps), _ptr(slots) if store_kv else 0, _ptr(q_out),
+         _ptr(k_pages) if store_kv else 0, _ptr(v_pages) if store_kv else 0, bs, int(bool(store_kv)), T, _stream())  # fmt: skip
+
+
+def sigmoid_gate_heads(heads, vdim, gate, gate_off, scale, out, out_off) -> None:
+    """out[t, out_off + h * vdim + j] = scale * sigmoid(gate[t, gate_off + h * vdim + j]) * heads[t, h, j], j < vdim."""
+    _check(heads, "heads", (F32, BF16), (None, None, None))
+    T, H, Dp = heads.shape
+    _check(gate, "gate", heads.dtype, (T, None))
+    _check(out, "out", heads.dtype, (T, None))
+    if vdim > Dp or gate_off < 0 or gate_off + H * vdim > gate.shape[1] or out_off < 0 or out_off + H * vdim > out.shape[1]:
+        raise KernelError("sigmoid_gate_heads: columns outside the gate or the output")
+    call("as_sigmoid_gate_heads", _ptr(heads), _DT[heads.dtype], H, vdim, Dp, _ptr(gate), gate.shape[1], gate_off,
+         float(scale), _ptr(out), out.shape[1], out_off, T, _stream())  # fmt: skip
+
+
+# ---- mixers with a fixed-size state --------------------------------------------------------------------
+
+
+def _check_rows(step_rows, num_tokens):
+    tok_row, row_first, row_len, row_start, row_slots = step_rows
+    _check(row_first, "row_first", I32, (None,))
+    R = row_first.shape[0]
+    for name, t in (("row_len", row_len), ("row_start", row_start), ("row_slots", row_slots)):
+        _check(t, name, I32, (R,))
+    if tok_row is not None:
+        _check(tok_row, "tok_row", I32, (num_tokens,))
+    elif R < num_tokens:
+        raise KernelError("tokens that are their own rows need as many rows")
+    return R
+
+
+def _vector_dtype(proj_dtype, *vectors):
+    dtypes = {v.dtype for v in vectors if v is not None}
+    if len(dtypes) > 1:
+        raise KernelError(f"the small tensors of one part come in one dtype, not {sorted(map(str, dtypes))}")
+    dtype = dtypes.pop() if dtypes else proj_dtype
+    if dtype not in _DT or (proj_dtype == F32 and dtype != F32):
+        raise KernelError(f"small tensors in {dtype} do not go with a projection in {proj_dtype}")
+    return dtype
+
+
+CONV_MAX_TAPS = 8
+
+
+def short_conv(proj, col0, weight, history, step_rows, out, in_bias=None, bias=None, silu=False, writes=True) -> None:
+    """Causal convolution per channel over each row's tokens: out[t, c] = act(sum_i weight[c, i] * in[t - (taps-1-i), c]
+    + bias[c]) with in = proj[:, col0 + c] + in_bias[c], zeros before a sequence, and before a row the last taps - 1
+    inputs of its request from history [slots, taps - 1, C] (fp32), which then moves on by the row (`writes`).
+    step_rows: (tok_row or None, row_first, row_len, row_start, row_slots).  out fp32 [T, C]."""
+    _check(proj, "proj", (F32, BF16), (None, None))
+    T, ld = proj.shape
+    _check(weight, "weight", (F32, BF16), (None, None))
+    C, taps = weight.shape
+    if not 1 <= taps <= CONV_MAX_TAPS or col0 < 0 or col0 + C > ld:
+        raise KernelError(f"short_conv: {taps} taps (1 to {CONV_MAX_TAPS}) or columns {col0}:{col0 + C} of {ld}")
+    w_dtype = _vector_dtype(proj.dtype, weight, in_bias, bias)
+    for name, b in (("in_bias", in_bias), ("bias", bias)):
+        if b is not None:
+            _check(b, name, w_dtype, (C,))
+    _check(out, "out", F32, (T, C))
+    R = _check_rows(step_rows, T)
+    _check(history, "history", F32, (None, max(taps - 1, 0), C) if taps > 1 else None)
+    tok_row, row_first, row_len, row_start, row_slots = step_rows
+    call("as_short_conv", _ptr(proj), _DT[proj.dtype], ld, col0, C, _ptr(in_bias), _ptr(weight), _ptr(bias),
+         _DT[w_dtype], taps, int(bool(silu)), _ptr(history), _ptr(tok_row), _ptr(row_first), _ptr(row_len),
+         _ptr(row_start), _ptr(row_slots), _ptr(out), T, R, int(bool(writes)), _stream())  # fmt: skip
+
+
+def delta_prepare(qkv, num_kv_heads, dim, num_heads, proj, b_off, a_off, a_log, dt_bias, beta, decay) -> None:
+    """In place on qkv fp32 [T, C] (G query heads, then G key heads, `dim` wide each, then the values): queries and
+    keys become unit vectors (x / sqrt(sum x^2 + 1e-6)), the queries also times dim^(-1/2).  beta [T, H] =
+    sigmoid(proj[:, b_off + h]); decay [T, H] = exp(-exp(a_log[h]) * softplus(proj[:, a_off + h] + dt_bias[h]))."""
+    _check(qkv, "qkv", F32, (None, None))
+    T, C = qkv.shape
+    G, H = num_kv_heads, num_heads
+    _check(proj, "proj", (F32, BF16), (T, None))
+    ld = proj.shape[1]
+    if C < 2 * G * dim or min(b_off, a_off) < 0 or max(b_off, a_off) + H > ld:
+        raise KernelError("delta_prepare: heads outside the convolution's channels or the projection's columns")
+    w_dtype = _vector_dtype(proj.dtype, a_log, dt_bias)
+    _check(a_log, "a_log", w_dtype, (H,))
+    _check(dt_bias, "dt_bias", w_dtype, (H,))
+    _check(beta, "beta", F32, (T, H))
+    _check(decay, "decay", F32, (T, H))
+    call("as_delta_prepare", _ptr(qkv), C, G, dim, H, _ptr(proj), _DT[proj.dtype], ld, b_off, a_off, _ptr(a_log),
+         _ptr(dt_bias), _DT[w_dtype], _ptr(beta), _ptr(decay), T, _stream())  # fmt: skip
+
+
+def delta_scan(qkv, num_kv_heads, dim, num_heads, vdim, beta, decay, state, step_rows, out, writes=True) -> None:
+    """The gated delta rule over each row's tokens, per head h (keys and queries of head h // (H / G)):
+    S <- decay S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.  state fp32 [slots, H, dim, vdim]; a row
+    that starts at position 0 starts from zero.  qkv as `delta_prepare` left it; out fp32 [T, H, vdim]."""
+    _check(qkv, "qkv", F32, (None, None))
+    T, C = qkv.shape
+    G, H = num_kv_heads, num_heads
+    if H % G or C != 2 * G * dim + H * vdim:
+        raise KernelError(f"delta_scan: {C} channels are not 2 x {G} x {dim} + {H} x {vdim}")
+    _check(beta, "beta", F32, (T, H))
+    _check(decay, "decay", F32, (T, H))
+    _check(state, "state", F32, (None, H, dim, vdim))
+    _check(out, "out", F32, (T, H, vdim))
+    R = _check_rows((None, *step_rows[1:]), 0)
+    _, row_first, row_len, row_start, row_slots = step_rows
+    call("as_delta_scan", _ptr(qkv), C, G, dim, H, vdim, _ptr(beta), _ptr(decay), _ptr(state), _ptr(row_first),
+         _ptr(row_len), _ptr(row_start), _ptr(row_slots), int(bool(writes)), _ptr(out), R, _stream())  # fmt: skip
+
+
+def delta_finish(o, weight, eps, proj, g_off, act) -> None:
+    """act[t, h * vdim + j] = o[t, h, j] / rms(o[t, h]) * weight[j] * silu(proj[t, g_off + h * vdim + j])."""
+    _check(o, "o", F32, (None, None, None))
+    T, H, vdim = o.shape
+    _check(proj, "proj", (F32, BF16), (T, None))
+    if g_off < 0 or g_off + H * vdim > proj.shape[1]:
+        raise KernelError("delta_finish: the gate lies outside the projection's columns")
+    w_dtype = _vector_dtype(proj.dtype, weight)
+    _check(weight, "weight", w_dtype, (vdim,))
+    _check(act, "act", proj.dtype, (T, H * vdim))
+    call("as_delta_finish", _ptr(o), H, vdim, _ptr(weight), _DT[w_dtype], float(eps), _ptr(proj), _DT[proj.dtype],
+         proj.shape[1], g_off, _ptr(act), T, _stream())  # fmt: skip
+
+
+def rglru_gates(u, ra, ra_bias, ri, ri_bias, lam, c, a_out, x_out) -> None:
+    """The two gates of a gated linear recurrence, per block of channels (ra, ri [blocks, bw, bw], out x in):
+    r = sigmoid(ra u_b + ra_bias), i = sigmoid(ri u_b + ri_bias); a_out = exp(-c r softplus(lam)),
+    x_out = sqrt(1 - a^2) i u.  u, a_out, x_out fp32 [T, width]."""
+    _check(u, "u", F32, (None, None))
+    T, width = u.shape
+    _check(ra, "ra", (F32, BF16), (None, None, None))
+    blocks, bw, _ = ra.shape
+    if blocks * bw != width or ra.shape[2] != bw:
+        raise KernelError(f"rglru_gates: {blocks} blocks of {tuple(ra.shape[1:])} do not make {width} channels")
+    _check(ri, "ri", ra.dtype, (blocks, bw, bw))
+    for name, v in (("ra_bias", ra_bias), ("ri_bias", ri_bias), ("lam", lam)):
+        _check(v, name, ra.dtype)
+        if v.numel() != width:
+            raise KernelError(f"{name} has {v.numel()} entries for {width} channels")
+    _check(a_out, "a_out", F32, (T, width))
+    _check(x_out, "x_out", F32, (T, width))
+    call("as_rglru_gates", _ptr(u), width, blocks, _ptr(ra), _ptr(ra_bias), _ptr(ri), _ptr(ri_bias), _ptr(lam),
+         _DT[ra.dtype], float(c), _ptr(a_out), _ptr(x_out), T, _stream())  # fmt: skip
+
+
+def rglru_scan(a, x, proj, y_off, y_bias, scale, state, step_rows, out, out_off, writes=True) -> None:
+    """S = a S + x per channel over each row's tokens (state fp32 [slots, width]; from zero at position 0);
+    out[t, out_off + c] = scale * S * gelu_tanh(proj[t, y_off + c] + y_bias[c])."""
+    _check(a, "a", F32, (None, None))
+    T, width = a.shape
+    _check(x, "x", F32, (T, width))
+    _check(proj, "proj", (F32, BF16), (T, None))
+    _check(out, "out", proj.dtype, (T, None))
+    if y_off < 0 or y_off + width > proj.shape[1] or out_off < 0 or out_off + width > out.shape[1]:
+        raise KernelError("rglru_scan: columns outside the projection or the output")
+    w_dtype = _vector_dtype(proj.dtype, y_bias)
+    if y_bias is not None:
+        _check(y_bias, "y_bias", w_dtype, (width,))
+    _check(state, "state", F32, (None, width))
+    R = _check_rows((None, *step_rows[1:]), 0)
+    _, row_first, row_len, row_start, row_slots = step_rows
+    call("as_rglru_scan", _ptr(a), _ptr(x), width, _ptr(proj), _DT[proj.dtype], proj.shape[1], y_off, _ptr(y_bias),
+         _DT[w_dtype], float(scale), _ptr(state), _ptr(row_first), _ptr(row_len), _ptr(row_start), _ptr(row_slots),
+         int(bool(writes)), _ptr(out), out.shape[1], out_off, R, _stream())  # fmt: skip
+
+
+# ---- experts ------------------------------------------------------------------------------------------
+
+MOE_TILE = 16
+MOE_MAX_EXPERTS = 1024
+
+
+class ExpertRoute:
+    """Where a step's (token, chosen expert) pairs stand once sorted by expert: what the grouped products read."""
+
+    __slots__ = ("order", "tiles", "counts", "max_tiles", "top", "num_tokens")
+
+    def __init__(self, num_tokens: int, top: int, experts: int, device):
+        pairs = num_tokens * top
+        self.max_tiles = -(-pairs // MOE_TILE) + experts
+        self.order = torch.empty(max(pairs, 1), dtype=I32, device=device)
+        self.tiles = torch.empty((self.max_tiles, 3), dtype=I32, device=device)
+        self.counts = torch.empty(1, dtype=I32, device=device)
+        self.top, self.num_tokens = top, num_tokens
+
+
+def moe_route_table(token_ids, table, experts: int) -> ExpertRoute:
+    """Routes by a table [vocab, top] int32 that names every token id's experts."""
+    _check(token_ids, "token_ids", I32, (None,))
+    _check(table, "table", I32, (None, None))
+    vocab, top = table.shape
+    if not 1 <= experts <= MOE_MAX_EXPERTS:
+        raise KernelError(f"routing sorts up to {MOE_MAX_EXPERTS} experts, not {experts}")
+    route = ExpertRoute(token_ids.shape[0], top, experts, token_ids.device)
+    call("as_moe_route_table", _ptr(token_ids), _ptr(table), vocab, top, experts, token_ids.shape[0], _ptr(route.order),
+         _ptr(route.tiles), _ptr(route.counts), route.max_tiles, _stream())  # fmt: skip
+    return route
+
+
+def moe_gemm(a, w, route: ExpertRoute, out, gated: bool, per_token: bool) -> None:
+    """The product of every pair's input with its expert's matrix, w [experts, N_w, K].  per_token: a [T, K] holds
+    a row per token (all of a token's pairs read it), else a row per pair.  gated: N_w = 2 N, out[p] =
+    silu(w[e, :N] a) * (w[e, N:] a); else out[p] = w[e] a.  out [pairs, N]: a's dtype, or fp32."""
+    _check(a, "a", (F32, BF16), (None, None))
+    K = a.shape[1]
+    pairs = route.num_tokens * route.top
+    if a.shape[0] != (route.num_tokens if per_token else pairs):
+        raise KernelError(f"moe_gemm: {a.shape[0]} input rows for {route.num_tokens} tokens of {route.top} experts")
+    _check(w, "w", a.dtype, (None, None, K))
+    N = w.shape[1] // 2 if gated else w.shape[1]
+    if gated and w.shape[1] % 2:
+        raise KernelError("moe_gemm: gate and up rows come in equal numbers")
+    _check(out, "out", (a.dtype, F32), (pairs, N))
+    if a.dtype == BF16 and K % 8:
+        raise KernelError("moe_gemm: bf16 rows are read 16 bytes at a time (width % 8 == 0)")
+    if gated and out.dtype != a.dtype:
+        raise KernelError("moe_gemm: the gated product's result has the inputs' dtype")
+    call("as_moe_gemm", _ptr(a), _DT[a.dtype], route.top if per_token else 1, _ptr(w), N, K, int(bool(gated)),
+         _ptr(route.order), _ptr(route.tiles), _ptr(route.counts), route.max_tiles, _ptr(out), _DT[out.dtype], _stream())  # fmt: skip
+
+
+def moe_combine(pair_out, top: int, weight: float, out) -> None:
+    """out[t] = sum_j weight * pair_out[t * top + j]; pair_out fp32 [T * top, N]."""
+    _check(out, "out", (F32, BF16), (None, None))
+    T, N = out.shape
+    _check(pair_out, "pair_out", F32, (T * top, N))
+    call("as_moe_combine", _ptr(pair_out), top, float(weight), N, _ptr(out), _DT[out.dtype], T, _stream())

@@ -72,21 +72,32 @@ class DecoderModel:
 
     # ---- caches ---------------------------------------------------------------------
     def cache_requests(self) -> dict:
-        """cache id -> what the mixer writing it asks of the cache manager."""
+        """cache id -> what the mixer writing it asks of the cache manager.  A mixer that keeps several
+        things (`Mixer.cache_request` returns a dict) has one entry per name, under the id (cache id, name)."""
+        def asked(mixer) -> dict:
+            req = mixer.cache_request()
+            if req is None:
+                return {}
+            return dict(req) if isinstance(req, dict) else {None: req}
+
+        def ident(cid, name):
+            return cid if name is None else (cid, name)
+
         requests = {}
         for i, r in enumerate(self.plan.run):
             cid = self.plan.cache_id(i)
-            req = self.blocks[r.layer].parts()["mixer"].cache_request()
-            if req is None:
+            if not r.writes:
                 continue
-            if r.writes:
-                if cid in requests and requests[cid] != req:
+            for name, req in asked(self.blocks[r.layer].parts()["mixer"]).items():
+                key = ident(cid, name)
+                if key in requests and requests[key] != req:
                     raise ValueError(f"runs sharing cache {cid} ask for different caches")
-                requests[cid] = req
+                requests[key] = req
         for i, r in enumerate(self.plan.run):
             cid = self.plan.cache_id(i)
-            if self.blocks[r.layer].parts()["mixer"].cache_request() is not None and cid not in requests:
-                raise ValueError(f"run {i} reads cache {cid}, which no run writes")
+            for name in asked(self.blocks[r.layer].parts()["mixer"]):
+                if ident(cid, name) not in requests:
+                    raise ValueError(f"run {i} reads cache {cid}, which no run writes")
         return requests
 
     # ---- one pass ---------------------------------------------------------------------

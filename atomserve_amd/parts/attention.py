@@ -128,24 +128,29 @@ class Attention(Mixer):
         return y
 
     def attend(self, q, out, step, cache) -> None:
-        s = self.spec
-        # fp32, and shapes the prefill kernel does not take: every token is a single query.
-        # Otherwise short rows are single queries and long rows go through the prefill kernel.
-        if step.decode_only:  # token t is row t: the kernels need no maps from one to the other
-            ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, None,
-                                  cache.block_tables, out, s.scale, s.window, step.max_context)  # fmt: skip
-            return
-        if not ops.attn_prefill_supported(self.env.dtype, s.head_dim, cache.block_size):
-            ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, step.tok_row,
-                                  cache.block_tables, out, s.scale, s.window, step.max_context)  # fmt: skip
-            return
-        rows = step.split(self.row_split())
-        if rows.num_short_tokens:
-            ops.attn_single_query(q, cache.k_pages, cache.v_pages, rows.short_tokens, step.positions, step.tok_row,
-                                  cache.block_tables, out, s.scale, s.window, rows.max_short_context)  # fmt: skip
-        if rows.num_long_tiles:
-            ops.attn_prefill(q, cache.k_pages, cache.v_pages, rows.long_tiles, cache.block_tables, out, s.scale,
-                             s.window, step.max_context, tile_keys=rows.tile_keys)  # fmt: skip
+        attend(q, out, step, cache, self.spec.scale, self.spec.window, self.row_split())
+
+
+def attend(q, out, step, cache, scale: float, window: int, split) -> None:
+    """Attention of a step's queries q [T, H, D] over the pages of `cache` (which hold the step's own keys
+    already) into out [T, H, D]; `split`: the (short, tile) under which the step sorted its rows for this."""
+    # fp32, and shapes the prefill kernel does not take: every token is a single query.
+    # Otherwise short rows are single queries and long rows go through the prefill kernel.
+    if step.decode_only:  # token t is row t: the kernels need no maps from one to the other
+        ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, None,
+                              cache.block_tables, out, scale, window, step.max_context)  # fmt: skip
+        return
+    if not ops.attn_prefill_supported(q.dtype, q.shape[2], cache.block_size):
+        ops.attn_single_query(q, cache.k_pages, cache.v_pages, step.all_tokens, step.positions, step.tok_row,
+                              cache.block_tables, out, scale, window, step.max_context)  # fmt: skip
+        return
+    rows = step.split(split)
+    if rows.num_short_tokens:
+        ops.attn_single_query(q, cache.k_pages, cache.v_pages, rows.short_tokens, step.positions, step.tok_row,
+                              cache.block_tables, out, scale, window, rows.max_short_context)  # fmt: skip
+    if rows.num_long_tiles:
+        ops.attn_prefill(q, cache.k_pages, cache.v_pages, rows.long_tiles, cache.block_tables, out, scale,
+                         window, step.max_context, tile_keys=rows.tile_keys)  # fmt: skip
 
 
 register("mixer", "attention", Attention)

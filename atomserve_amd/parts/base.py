@@ -7,8 +7,8 @@ Kinds of parts:
   norm          forward(x, delta, rows) -> normalised rows, optionally adding `delta`
                 into the fp32 residual stream first
   position      prepare(step) once per step; mixers ask it for what their kernel needs
-  mixer         forward(h, step, cache) -> [T, hidden]; says which cache it wants
-                through `cache_request()`
+  mixer         forward(h, step, cache) -> [T, hidden]; says which cache (or caches) it
+                wants through `cache_request()`
   feed_forward  forward(h, step) -> [T, hidden]
   arrangement   runs one layer: owns the order of norms, mixer, feed-forward and
                 residual sums
@@ -129,6 +129,14 @@ class SplitSums:
         self.sums = sums
 
 
+class DeltaSum:
+    """Outputs of several parts that read the same stream, all still to be added into it: a norm that
+    takes one adds them up in fp32 on its way (`parts`: tensors [T, hidden] in the compute dtype)."""
+
+    def __init__(self, parts):
+        self.parts = tuple(p for p in parts if p is not None)
+
+
 class Mixer(Part):
     # Two optional shortcuts an arrangement may take with a part that declares them:
     # takes_pending_norm: `h` may arrive as a PendingNorm instead of normalised rows;
@@ -140,6 +148,10 @@ class Mixer(Part):
     adds_to_residual = False
 
     def cache_request(self) -> Optional[Any]:
+        """What this mixer keeps between steps: a `PagedCacheRequest`, a `StateCacheRequest`, None, or a
+        dict name -> request for a mixer that keeps several things (pages of keys and values beside a
+        recurrent state, a state beside a convolution's last inputs); it is then handed a dict of views
+        under the same names."""
         return None
 
     def row_split(self) -> Optional[tuple]:
@@ -233,4 +245,4 @@ def build(family: str, spec: Any, env: BuildEnv):
 
 
 def _load_builtin() -> None:
-    from atomserve_amd.parts import attention, block, mlp, norm, rope  # noqa: F401
+    from atomserve_amd.parts import attention, block, experts, mlp, norm, recurrent, rope  # noqa: F401

@@ -1,6 +1,7 @@
 """Arrangements: how one layer orders its norms, mixer, feed-forward and residual sums.
 
-"prenorm":  x += mixer(norm(x));  x += ffn(norm(x))   (reference atomserve/model.py:378-382)
+"prenorm":    x += mixer(norm(x));  x += ffn(norm(x))   (reference atomserve/model.py:378-382)
+"two_norms":  x += mixer(norm1(x)) + ffn(norm2(x)), both parts reading the same x through a norm each
 
 The residual stream `x` is fp32 in both precisions.  A part's output is not added at
 once: it travels as the pending `delta` to the next norm, whose kernel adds it into
@@ -9,7 +10,7 @@ products around them instead: a part's last product adds into `x` and leaves the
 pending (`Norm.absorb`), and the next part's first product finishes it (`PendingNorm`).
 """
 
-from atomserve_amd.parts.base import Arrangement, PendingNorm, build, register
+from atomserve_amd.parts.base import Arrangement, DeltaSum, PendingNorm, build, register
 
 
 class PreNormBlock(Arrangement):
@@ -44,3 +45,46 @@ class PreNormBlock(Arrangement):
 
 
 register("arrangement", "prenorm", PreNormBlock)
+
+
+class TwoNormsBlock(Arrangement):
+    """x += mixer(mixer_norm(x)) + ffn(ffn_norm(x)): the two parts read the same stream, each through a norm of
+    its own.  Both outputs travel on as one pending `DeltaSum`; the kernel that starts the next layer adds them
+    into the stream (in fp32) and takes both of that layer's norms from one root mean square.  A layer without
+    a feed-forward (spec.ffn None) is the mixer alone."""
+
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        self.mixer_norm = build("norm", spec.mixer_norm, env)
+        self.mixer = build("mixer", spec.mixer, env)
+        self.ffn_norm = self.ffn = None
+        if spec.ffn is not None:
+            self.ffn_norm = build("norm", spec.ffn_norm, env)
+            self.ffn = build("feed_forward", spec.ffn, env)
+        self.shared_kernel = self.ffn is not None and hasattr(self.mixer_norm, "with_sibling") and \
+            type(self.mixer_norm) is type(self.ffn_norm) and spec.mixer_norm.eps == spec.ffn_norm.eps  # fmt: skip
+
+    def parts(self) -> dict:
+        parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        if self.ffn is not None:
+            parts.update(ffn_norm=self.ffn_norm, ffn=self.ffn)
+        return parts
+
+    def first_norm(self):
+        return None  # nothing is left pending inside a product for this layer: it takes a sum of outputs
+
+    def forward(self, x, delta, step, cache, next_norm=None):
+        if isinstance(delta, PendingNorm):
+            raise ValueError("a layer of two norms takes pending outputs, not a norm left pending in a product")
+        if self.shared_kernel:
+            h1, h2 = self.mixer_norm.with_sibling(self.ffn_norm, x, delta)
+        else:
+            h1 = self.mixer_norm.forward(x, delta)
+            h2 = self.ffn_norm.forward(x) if self.ffn is not None else None
+        mixed = self.mixer.forward(h1, step, cache)
+        if self.ffn is None:
+            return mixed
+        return DeltaSum((mixed, self.ffn.forward(h2, step)))
+
+
+register("arrangement", "two_norms", TwoNormsBlock)

@@ -6,7 +6,7 @@ pre-norm layer is fused into the same kernel: the fp32 residual stream `x` recei
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import Norm, PendingNorm, SplitSums, WeightDecl, register
+from atomserve_amd.parts.base import DeltaSum, Norm, PendingNorm, SplitSums, WeightDecl, register
 
 
 class PendingRMSNorm(PendingNorm):
@@ -53,11 +53,32 @@ class RMSNorm(Norm):
         rows: int32 row selection, or None for all rows.  Returns [rows, size], compute dtype."""
         n_out = x.shape[0] if rows is None else rows.shape[0]
         out = torch.empty((n_out, self.spec.size), dtype=self.env.dtype, device=x.device)
-        if isinstance(delta, SplitSums):
+        if isinstance(delta, DeltaSum):
+            self.with_sibling(None, x, delta, rows, update_residual, out)
+        elif isinstance(delta, SplitSums):
             ops.rmsnorm(x, self.weight, self.spec.eps, out, rows=rows, update_x=update_residual, split_sums=delta.sums)
         else:
             ops.rmsnorm(x, self.weight, self.spec.eps, out, delta=delta, rows=rows, update_x=update_residual)
         return out
+
+
+    def with_sibling(self, other, x, delta=None, rows=None, update_residual=True, out=None):
+        """This norm and `other` (an RMSNorm of the same size and eps, or None) of the same stream in one
+        kernel: x += delta (a tensor, a `DeltaSum` of up to two, or None), the root mean square taken once.
+        Returns (this norm's rows, the other's or None)."""
+        parts = delta.parts if isinstance(delta, DeltaSum) else (() if delta is None else (delta,))
+        if len(parts) > 2 or any(not isinstance(p, torch.Tensor) for p in parts):
+            raise ValueError("a norm adds up to two pending outputs (tensors) into the stream")
+        if other is not None and (other.spec.size, other.spec.eps) != (self.spec.size, self.spec.eps):
+            raise ValueError("two norms of one stream share a kernel only with one size and one eps")
+        n_out = x.shape[0] if rows is None else rows.shape[0]
+        if out is None:
+            out = torch.empty((n_out, self.spec.size), dtype=self.env.dtype, device=x.device)
+        out2 = torch.empty_like(out) if other is not None else None
+        ops.rmsnorm_multi(x, self.weight, other.weight if other is not None else None, self.spec.eps, out, out2,
+                          delta1=parts[0] if parts else None, delta2=parts[1] if len(parts) > 1 else None, rows=rows,
+                          update_x=update_residual)  # fmt: skip
+        return out, out2
 
 
 register("norm", "rmsnorm", RMSNorm)

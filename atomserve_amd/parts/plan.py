@@ -53,15 +53,94 @@ class GatedMLPSpec:
 
 
 @dataclass(frozen=True)
+class ShortConvSpec:
+    """Causal convolution per channel over the last `taps` tokens (the last tap is the current token's)."""
+
+    taps: int
+
+
+@dataclass(frozen=True)
+class DeltaRuleSpec:
+    """Gated delta rule: per head a state [key_dim, value_dim] that decays, is corrected towards the
+    token's value along its key and is read along its query; q, k, v pass a short convolution and silu,
+    q and k become unit vectors (eps inside the root), the output is normed per head and gated.
+    num_kv_heads heads of q and k serve num_heads heads of v."""
+
+    kind: str  # "delta_rule"
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    conv: ShortConvSpec
+    out_norm_eps: float  # of the RMS norm of every head's output
+    unit_eps: float = 1e-6  # inside the root of the unit norms
+
+
+@dataclass(frozen=True)
+class GatedAttentionSpec:
+    """Softmax attention whose concatenated heads are multiplied by sigmoid(gate(h)) before the output
+    projection.  Keys and queries are `key_dim` wide, values `value_dim`; no position encoding."""
+
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    qk_norm: Optional[NormSpec]
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class LinearRecurrenceSpec:
+    """Real-gated linear recurrent unit: S = a S + sqrt(1 - a^2) i u with a = exp(-decay_scale r softplus(lam)),
+    the gates r and i from block-diagonal matrices on u = conv(x(h)); the output is S * gelu(y(h))."""
+
+    width: int
+    blocks: int
+    conv: ShortConvSpec
+    decay_scale: float = 8.0
+
+
+@dataclass(frozen=True)
+class SideBySideSpec:
+    """Two mixers that read the same input; their outputs are added with a weight each, inside one
+    output projection: left_scale * attention + right_scale * recurrence."""
+
+    kind: str  # "side_by_side"
+    hidden_size: int
+    left: GatedAttentionSpec
+    right: LinearRecurrenceSpec
+    left_scale: float
+    right_scale: float
+
+
+@dataclass(frozen=True)
+class TableExpertsSpec:
+    """Gated feed-forward experts of which every token uses `top`, named by a table indexed with the
+    token id; each chosen expert weighs 1 / top."""
+
+    kind: str  # "table_experts"
+    hidden_size: int
+    intermediate_size: int
+    num_experts: int
+    top: int
+    vocab_size: int
+    activation: str  # "silu"
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: a mixer and a feed-forward with their norms, and how they are arranged.
-    arrangement "prenorm": x += mixer(norm(x)); x += ffn(norm(x))."""
+    arrangement "prenorm": x += mixer(norm(x)); x += ffn(norm(x)).
+    arrangement "two_norms": x += mixer(mixer_norm(x)) + ffn(ffn_norm(x)), both of the same x
+    (ffn and ffn_norm None: the mixer alone)."""
 
     arrangement: str
     mixer: Any
     mixer_norm: NormSpec
     ffn: Any
-    ffn_norm: NormSpec
+    ffn_norm: Optional[NormSpec]
 
 
 @dataclass(frozen=True)

@@ -1,7 +1,8 @@
 """Random weights from a configuration and a seed, as a model folder or in memory.
 
 One seeded generator draws every tensor in the order the architecture lists them:
-matrices N(0, std), gains 1 + N(0, gain_std).  Values are drawn in fp32 and rounded
+matrices and biases N(0, std), gains 1 + N(0, gain_std), logarithms of rates N(0, 0.5), tables
+of experts as rows of distinct expert numbers.  Values are drawn in fp32 and rounded
 to the storage dtype, so a bfloat16 folder read back in float32 holds the same numbers.
 """
 
@@ -19,8 +20,18 @@ def random_checkpoint(arch, config, seed: int, dtype=torch.bfloat16, device="cpu
     gen.manual_seed(seed)
     out = {}
     for name, (shape, role) in arch.checkpoint_shapes(config).items():
+        if role.startswith("expert_table:"):  # every row names distinct experts
+            experts = int(role.split(":")[1])
+            keys = torch.rand((shape[0], experts), generator=gen, device=device)
+            out[name] = keys.argsort(dim=1)[:, : shape[1]].to(torch.int32).contiguous()
+            continue
         t = torch.randn(tuple(shape), generator=gen, device=device, dtype=torch.float32)
-        t = t.mul_(gain_std).add_(1.0) if role == "vector" else t.mul_(std)
+        if role == "vector":
+            t = t.mul_(gain_std).add_(1.0)
+        elif role == "log_rate":
+            t = t.mul_(0.5)
+        else:
+            t = t.mul_(std)
         out[name] = t.to(dtype)
     return out
 
