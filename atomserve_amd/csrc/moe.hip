@@ -3,14 +3,15 @@
 // Which experts a token uses is decided on the GPU (a table indexed by the token id here), so a step
 // never waits for the host and can be replayed as a graph.  A (token, chosen expert) is a "pair":
 // pair p = token * top + choice.  `moe_route` sorts the pairs by expert and cuts every expert's run
-// into tiles of 16; the two grouped products then take one workgroup per (tile, 64 outputs): the first
+// into tiles of up to 64; the two grouped products then take one workgroup per (tile, 64 outputs): the first
 // applies act(gate) * up on the way out, the second writes every pair's output where the pair stands
 // (so the outputs of a token's experts lie side by side), and `moe_combine` adds them up with their
 // weights.  A pair's result does not depend on what else is in the step: every output is a dot product
 // over the whole width in a fixed order.
 #include "common.h"
 
-#define MOE_TILE 16      // pairs of one expert that a workgroup takes
+#define MOE_TILE 64      // pairs of one expert that a workgroup takes (four column tiles of 16)
+#define MOE_KC 128       // inputs per round: the tile's activations of a round meet in LDS
 #define MOE_STRIP 64     // outputs that a workgroup takes: four waves of 16
 #define MOE_MAX_EXPERTS 1024
 
@@ -19,7 +20,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 // ---- routing ------------------------------------------------------------------------------------
 // table [vocab, top] int32: the experts of every token id.  order [P]: the pairs sorted by expert;
-// tiles [max_tiles, 3]: (expert, first place in `order`, count <= 16); counts[0] = number of tiles.
+// tiles [max_tiles, 3]: (expert, first place in `order`, count <= 64); counts[0] = number of tiles.
 // One workgroup; the order of pairs within an expert is whatever the atomics make it, which no
 // result depends on.
 __global__ __launch_bounds__(1024) void moe_route_table_kernel(const int* __restrict__ token_ids,
@@ -80,59 +81,96 @@ extern "C" int as_moe_route_table(const int* token_ids, const int* table, int vo
 // GATED: N_w = 2 N, rows 0..N-1 the gate, N..2N-1 the up projection; out[p, n] = silu(gate) * up.
 // else:  out[p, n] = the product.  out has a row per pair.
 //
-// bf16: v_mfma_f32_16x16x32_bf16 with the weights as the A operand (16 rows of w) and the tile's 16
-// pairs as the B operand; a wave owns 16 outputs (and their up rows), walks K in steps of 32 and reads
-// both operands straight from memory, 16 bytes a lane.  Needs K % 8 == 0.
+// bf16: v_mfma_f32_16x16x32_bf16 with the weights as the A operand (16 rows of w) and 16 of the tile's
+// pairs as the B operand.  A wave owns 16 outputs (and their up rows) for all of the tile's pairs (up to
+// four column tiles of 16); the tile's activations are brought into LDS once per round of 128 inputs for
+// the four waves (rows padded by 16 bytes against bank conflicts), the weights go from memory straight
+// into registers, 16 bytes a lane.  Few pairs (a decode step) cost few products: column tiles beyond the
+// tile's count are skipped.  Needs K % 8 == 0.
 template <bool GATED, typename OutT>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restrict__ a, int a_div,
                                                             const bf16* __restrict__ w, int N, int K,
                                                             const int* __restrict__ order,
                                                             const int* __restrict__ tiles,
                                                             const int* __restrict__ counts, OutT* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) bf16 acts[MOE_TILE][MOE_KC + 8];
+  __shared__ int pair_of[MOE_TILE];
   const int tile = blockIdx.y;
   if (tile >= counts[0]) return;
   const int e = tiles[3 * tile], at = tiles[3 * tile + 1], cnt = tiles[3 * tile + 2];
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
   const int lr = lane & 15, lg = lane >> 4;
   const int n0 = blockIdx.x * MOE_STRIP + wave * 16;
-  if (n0 >= N) return;
-  const int pair = lr < cnt ? order[at + lr] : -1;  // this lane's column of the B operand
-  const bf16* arow = pair >= 0 ? a + (size_t)(pair / a_div) * K : nullptr;
+  const int col_tiles = (cnt + 15) >> 4;
+  if (threadIdx.x < MOE_TILE) pair_of[threadIdx.x] = threadIdx.x < cnt ? order[at + threadIdx.x] : -1;
+  __syncthreads();
   const int NW = GATED ? 2 * N : N;
   const bf16* wbase = w + (size_t)e * NW * K;
   const bool row_in = n0 + lr < N;
-  const bf16* wrow = wbase + (size_t)(n0 + lr) * K;
-  const bf16* urow = wbase + (size_t)(N + n0 + lr) * K;
-  floatx4 acc = {0.f, 0.f, 0.f, 0.f}, acc_up = {0.f, 0.f, 0.f, 0.f};
+  const bf16* wrow = wbase + (size_t)(row_in ? n0 + lr : 0) * K;
+  const bf16* urow = wbase + (size_t)(N + (row_in ? n0 + lr : 0)) * K;
+  floatx4 acc[4], acc_up[4];
+#pragma unroll
+  for (int ct = 0; ct < 4; ++ct) { acc[ct] = floatx4{0.f, 0.f, 0.f, 0.f}; acc_up[ct] = floatx4{0.f, 0.f, 0.f, 0.f}; }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const int k = k0 + lg * 8;
-    const bool k_in = k < K;
-    const bf16x8 av = (arow && k_in) ? *reinterpret_cast<const bf16x8*>(arow + k) : zero;
-    const bf16x8 wv = (row_in && k_in) ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc, 0, 0, 0);
-    if (GATED) {
-      const bf16x8 uv = (row_in && k_in) ? *reinterpret_cast<const bf16x8*>(urow + k) : zero;
-      acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv, av, acc_up, 0, 0, 0);
+  // staging: thread -> (row of the tile, 16-byte piece of the round): 64 rows x 16 pieces, four a thread
+  for (int k0 = 0; k0 < K; k0 += MOE_KC) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int piece = threadIdx.x + i * 256, row = piece >> 4, kk = (piece & 15) * 8;
+      if (row < col_tiles * 16) {
+        const int pair = pair_of[row];
+        const bf16x8 v = (pair >= 0 && k0 + kk < K) ? *reinterpret_cast<const bf16x8*>(a + (size_t)(pair / a_div) * K + k0 + kk) : zero;
+        *reinterpret_cast<bf16x8*>(&acts[row][kk]) = v;
+      }
+    }
+    bf16x8 wv[MOE_KC / 32], uv[MOE_KC / 32];
+#pragma unroll
+    for (int s = 0; s < MOE_KC / 32; ++s) {
+      const int k = k0 + s * 32 + lg * 8;
+      const bool in = row_in && k < K;
+      wv[s] = in ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
+      if (GATED) uv[s] = in ? *reinterpret_cast<const bf16x8*>(urow + k) : zero;
+    }
+    __syncthreads();
+    if (n0 < N) {
+#pragma unroll
+      for (int s = 0; s < MOE_KC / 32; ++s) {
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+          if (ct < col_tiles) {
+            const bf16x8 av = *reinterpret_cast<const bf16x8*>(&acts[ct * 16 + lr][s * 32 + lg * 8]);
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[s], av, acc[ct], 0, 0, 0);
+            if (GATED) acc_up[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv[s], av, acc_up[ct], 0, 0, 0);
+          }
+        }
+      }
     }
   }
-  // a lane holds outputs n0 + 4 lg + i (i < 4) of the pair in column lr
-  if (pair < 0) return;
+  // a lane holds outputs n0 + 4 lg + i (i < 4) of the pair in column lr of each column tile
+  if (n0 >= N) return;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int n = n0 + 4 * lg + i;
-    if (n >= N) continue;
-    float v = acc[i];
-    if (GATED) {
-      const float g = to_f32((bf16)acc[i]), u = to_f32((bf16)acc_up[i]);  // the two products rounded as if stored
-      v = g / (1.0f + expf(-g)) * u;
+  for (int ct = 0; ct < 4; ++ct) {
+    if (ct >= col_tiles) continue;
+    const int pair = pair_of[ct * 16 + lr];
+    if (pair < 0) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * lg + i;
+      if (n >= N) continue;
+      float v = acc[ct][i];
+      if (GATED) {
+        const float g = to_f32((bf16)acc[ct][i]), u = to_f32((bf16)acc_up[ct][i]);  // the two products rounded as if stored
+        v = g / (1.0f + expf(-g)) * u;
+      }
+      out[(size_t)pair * N + n] = from_f32<OutT>(v);
     }
-    out[(size_t)pair * N + n] = from_f32<OutT>(v);
   }
 }
 
-// fp32: plain multiply-add, every output one chain over k in order.  A thread owns an output and four
-// of the tile's sixteen pairs.
+// fp32: plain multiply-add, every output one chain over k in order.  A thread owns an output and, of every
+// sixteen of the tile's pairs in turn, four.
 template <bool GATED>
 __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(const float* __restrict__ a, int a_div,
                                                            const float* __restrict__ w, int N, int K,
@@ -147,30 +185,33 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(const float* __restri
   const int NW = GATED ? 2 * N : N;
   const float* wrow = w + ((size_t)e * NW + n) * K;
   const float* urow = w + ((size_t)e * NW + N + n) * K;
-  int pairs[4];
-  const float* arow[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int place = quarter * 4 + i;
-    pairs[i] = place < cnt ? order[at + place] : -1;
-    arow[i] = a + (size_t)(pairs[i] < 0 ? 0 : pairs[i] / a_div) * K;
-  }
-  float acc[4] = {0.f, 0.f, 0.f, 0.f}, acc_up[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int k = 0; k < K; ++k) {
-    const float wv = wrow[k], uv = GATED ? urow[k] : 0.f;
+  for (int base = 0; base < cnt; base += 16) {
+    int pairs[4];
+    const float* arow[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float av = arow[i][k];
-      acc[i] = fmaf(wv, av, acc[i]);
-      if (GATED) acc_up[i] = fmaf(uv, av, acc_up[i]);
+      const int place = base + quarter * 4 + i;
+      pairs[i] = place < cnt ? order[at + place] : -1;
+      arow[i] = a + (size_t)(pairs[i] < 0 ? 0 : pairs[i] / a_div) * K;
     }
-  }
+    if (pairs[0] < 0) continue;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f}, acc_up[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < K; ++k) {
+      const float wv = wrow[k], uv = GATED ? urow[k] : 0.f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if (pairs[i] < 0) continue;
-    float v = acc[i];
-    if (GATED) v = v / (1.0f + expf(-v)) * acc_up[i];
-    out[(size_t)pairs[i] * N + n] = v;
+      for (int i = 0; i < 4; ++i) {
+        const float av = arow[i][k];
+        acc[i] = fmaf(wv, av, acc[i]);
+        if (GATED) acc_up[i] = fmaf(uv, av, acc_up[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (pairs[i] < 0) continue;
+      float v = acc[i];
+      if (GATED) v = v / (1.0f + expf(-v)) * acc_up[i];
+      out[(size_t)pairs[i] * N + n] = v;
+    }
   }
 }
 

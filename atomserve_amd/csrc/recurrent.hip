@@ -231,6 +231,10 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
     return AS_BAD_SHAPE;
   int slices = 1;
   while ((dim + slices - 1) / slices > 64) slices *= 2;  // a lane keeps at most 64 rows of its column
+  // few rows and heads: narrower column groups (more slices of fewer rows) until the waves fill the GPU
+  while (slices < 8 && (dim + 2 * slices - 1) / (2 * slices) >= 8 &&
+         (long)num_rows * H * ((vdim + WAVE / slices - 1) / (WAVE / slices)) < 4L * compute_units())
+    slices *= 2;
   const int rows_per_lane = (dim + slices - 1) / slices;
   const int RPL = rows_per_lane <= 8 ? 8 : rows_per_lane <= 16 ? 16 : rows_per_lane <= 32 ? 32 : 64;
   const int CJ = WAVE / slices;
@@ -366,42 +370,49 @@ extern "C" int as_rglru_gates(const float* u, int width, int blocks, const void*
 
 // The scan: S = a S + x per channel, from zero at the start of a sequence; what leaves is
 // scale * S * gelu_tanh(y + y_bias) with y from proj [T, ld] at y_off, into out [T, ld_out] at out_off.
-// A thread owns a channel of a row; the loads of four tokens are asked for together.
+// A workgroup owns 64 channels of a row and cuts the row's tokens into SCAN_SEGS equal stretches, a wave
+// each: every wave first runs its stretch from zero (keeping the product of its decays and what it ends
+// with), the stretches' ends are chained in LDS in order, and every wave runs its stretch again from its
+// true start, now writing.  The chain of dependent steps is a row's length / 8 instead of its length.
+#define SCAN_SEGS 16
 template <typename T, typename W>
-__global__ void rglru_scan_kernel(const float* __restrict__ a, const float* __restrict__ x, int width,
-                                  const T* __restrict__ proj, int ld, int y_off, const W* __restrict__ y_bias,
-                                  float scale, float* __restrict__ state, const int* __restrict__ row_first,
-                                  const int* __restrict__ row_len, const int* __restrict__ row_start,
-                                  const int* __restrict__ row_slots, int writes, T* __restrict__ out, int ld_out,
-                                  int out_off) {
-  const int r = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= width) return;
+__global__ __launch_bounds__(64 * SCAN_SEGS) void rglru_scan_kernel(
+    const float* __restrict__ a, const float* __restrict__ x, int width, const T* __restrict__ proj, int ld, int y_off,
+    const W* __restrict__ y_bias, float scale, float* __restrict__ state, const int* __restrict__ row_first,
+    const int* __restrict__ row_len, const int* __restrict__ row_start, const int* __restrict__ row_slots, int writes,
+    T* __restrict__ out, int ld_out, int out_off) {
+  __shared__ float seg_a[SCAN_SEGS][WAVE], seg_b[SCAN_SEGS][WAVE];
+  const int lane = threadIdx.x & (WAVE - 1), seg = threadIdx.x / WAVE;
+  const int r = blockIdx.y, c = blockIdx.x * WAVE + lane;
+  const bool live = c < width;
   const int first = row_first[r], len = row_len[r], slot = row_slots[r];
-  float* mine = state + (size_t)(slot < 0 ? 0 : slot) * width + c;
-  float S = (row_start[r] > 0 && slot >= 0) ? *mine : 0.f;
-  const float yb = y_bias ? to_f32(y_bias[c]) : 0.f;
-  int j = 0;
-  for (; j + 4 <= len; j += 4) {
-    float av[4], xv[4], yv[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const size_t t = (size_t)first + j + k;
-      av[k] = a[t * width + c];
-      xv[k] = x[t * width + c];
-      yv[k] = to_f32(proj[t * ld + y_off + c]);
-    }
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      S = fmaf(av[k], S, xv[k]);
-      out[((size_t)first + j + k) * ld_out + out_off + c] = from_f32<T>(scale * S * gelu_tanhf_(yv[k] + yb));
+  const int per = (len + SCAN_SEGS - 1) / SCAN_SEGS;
+  const int lo = min(len, seg * per), hi = min(len, lo + per);
+  float A = 1.f, B = 0.f;
+  if (live) {
+#pragma unroll 4
+    for (int j = lo; j < hi; ++j) {
+      const size_t t = (size_t)first + j;
+      const float av = a[t * width + c];
+      B = fmaf(av, B, x[t * width + c]);
+      A *= av;
     }
   }
-  for (; j < len; ++j) {
+  seg_a[seg][lane] = A;
+  seg_b[seg][lane] = B;
+  __syncthreads();
+  if (!live) return;
+  float* mine = state + (size_t)(slot < 0 ? 0 : slot) * width + c;
+  float S = (row_start[r] > 0 && slot >= 0) ? *mine : 0.f;
+  for (int s = 0; s < seg; ++s) S = fmaf(seg_a[s][lane], S, seg_b[s][lane]);
+  const float yb = y_bias ? to_f32(y_bias[c]) : 0.f;
+#pragma unroll 4
+  for (int j = lo; j < hi; ++j) {
     const size_t t = (size_t)first + j;
     S = fmaf(a[t * width + c], S, x[t * width + c]);
     out[t * ld_out + out_off + c] = from_f32<T>(scale * S * gelu_tanhf_(to_f32(proj[t * ld + y_off + c]) + yb));
   }
-  if (writes && slot >= 0) *mine = S;
+  if (writes && slot >= 0 && seg == SCAN_SEGS - 1) *mine = S;  // the last stretch ends where the row ends
 }
 
 extern "C" int as_rglru_scan(const float* a, const float* x, int width, const void* proj, int dtype, int ld, int y_off,
@@ -410,8 +421,8 @@ extern "C" int as_rglru_scan(const float* a, const float* x, int width, const vo
                              int ld_out, int out_off, int num_rows, hipStream_t stream) {
   if (num_rows <= 0) return AS_OK;
   if (width <= 0 || num_rows > 65535 || ld < y_off + width || ld_out < out_off + width) return AS_BAD_SHAPE;
-  const int threads = width >= 1024 ? 256 : 64;
-  dim3 grid((width + threads - 1) / threads, num_rows);
+  const int threads = WAVE * SCAN_SEGS;
+  dim3 grid((width + WAVE - 1) / WAVE, num_rows);
 #define LAUNCH(T, W)                                                                                              \
   rglru_scan_kernel<T, W><<<grid, threads, 0, stream>>>(a, x, width, (const T*)proj, ld, y_off, (const W*)y_bias, \
                                                         scale, state, row_first, row_len, row_start, row_slots,  \

@@ -1224,7 +1224,7 @@ def rglru_scan(a, x, proj, y_off, y_bias, scale, state, step_rows, out, out_off,
 
 # ---- experts ------------------------------------------------------------------------------------------
 
-MOE_TILE = 16
+MOE_TILE = 64  # pairs of one expert that a workgroup of the grouped products takes
 MOE_MAX_EXPERTS = 1024
 
 

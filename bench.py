@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sizes 8b|0.6b|32b] [--batch B] [--context S]
     python bench.py --workload mixed --sizes 0.6b      (a continuous batch through the scheduler)
+    python bench.py --design dozusun [--widths 1024,2048,4096]   (Dozusun layers beside Qwen3 layers of equal size)
 
 A step is one decode step of the engine (scheduler, one pass over the GPU, sampling).
 Prints ONE JSON line: decoded tokens per second at batch 8 with 2,048-token contexts,
@@ -74,6 +75,11 @@ def parse_args():
                         "(half of them share their first 32), chunks of 512, 128 tokens decoded each, through the "
                         "scheduler from submission to the last token")  # fmt: skip
     p.add_argument("--chunk-budget", type=int, default=512, help="token budget of a step in the mixed workload")
+    p.add_argument("--design", choices=["qwen3", "dozusun"], default="qwen3",
+                   help="dozusun: prefill and decode throughput of random-weight Dozusun layers (an attention beside a "
+                        "gated linear recurrence, gated delta rules, dense and table-routed feed-forwards) at a few "
+                        "widths, beside Qwen3 layers of the same width, heads, depth and vocabulary")  # fmt: skip
+    p.add_argument("--widths", default="1024,2048,4096", help="stream widths of --design dozusun")
     p.add_argument("--profile", action="store_true",
                    help="also split the host's time of a decode step into schedule / pack / launch / sample / wait / "
                         "update (steps run one at a time meanwhile, none sent ahead), as the reference's "
@@ -155,6 +161,111 @@ def mixed_workload(args, model, config, full_layers: int) -> dict:
     }
 
 
+def dozusun_config(width: int, layers: int, vocab: int):
+    """Layers as a model of this design of that width would have them: heads of 128, a kv head to four query heads,
+    a window of 1,024, a recurrence as wide as the stream in blocks of 256 channels (128 at width 1,024), feed-forwards
+    three times the width, dense in the layers of the first kind and as 16 experts of a quarter of that (two to a token:
+    half a dense layer's arithmetic) in the layers of the second; the two kinds of layers in turn."""
+    from atomserve_amd.config.model_config import DozusunConfig
+
+    heads = width // 128
+    side = {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128**-0.5,
+                     "mask": {"size": 1024}},
+            "left_scale": 1.0, "right_scale": 1.0,
+            "right": {"width": width, "blocks": width // (256 if width >= 2048 else 128), "conv": 4}}  # fmt: skip
+    delta = {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 128, "vdim": 128, "conv": 4}
+    pair = [{"type": "parallel", "mixer": side, "mlp": {"kind": "dense", "ff": 3 * width}},
+            {"type": "delta", "mixer": delta, "mlp": {"kind": "moe", "expert": {"ff": 3 * width // 4},
+                                                       "router": {"experts": 16, "top": 2}}}]  # fmt: skip
+    return DozusunConfig.from_dict({"architecture": "Dozusun", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+                                    "layers": [pair[i % 2] for i in range(layers)]})  # fmt: skip
+
+
+def design_comparison(args) -> dict:
+    """Prefill of --prefill-tokens tokens and decode at batch 1 and --batch with --context tokens of context, for
+    Dozusun layers and for Qwen3 layers of equal width, heads, depth and vocabulary; random weights, the engine's own
+    entry point (scheduler, captured decode steps, sampling)."""
+    import torch
+
+    from atomserve_amd.config import EngineConfig, Qwen3Config
+    from atomserve_amd.config.registry import architecture_for
+    from atomserve_amd.engine.engine import create_engine
+    from atomserve_amd.engine.sequence import SamplingParams
+    from atomserve_amd.models.decoder import DecoderModel
+    from atomserve_amd.weights.loader import DictSource, bind_checkpoint
+    from atomserve_amd.weights.random_init import random_checkpoint
+
+    device, dtype = "cuda:0", (torch.bfloat16 if args.dtype == "bf16" else torch.float32)
+    layers, vocab, block = args.layers or 8, 32768, args.block_size
+    T, context, steps = args.prefill_tokens, args.context, max(16, min(args.steps, 64))
+    max_len = max(T, context) + steps + args.warmup + 2 * block
+    greedy = SamplingParams(temperature=0.0, max_tokens=100000, ignore_eos=True)
+
+    def measure(config) -> dict:
+        arch = architecture_for(config.to_dict())
+        model = DecoderModel(arch.build_plan(config), dtype, device)
+        bind_checkpoint(model, arch, config, DictSource(random_checkpoint(arch, config, seed=0, dtype=dtype, device=device)))
+        batches = sorted({1, args.batch})
+        engine = create_engine(model, EngineConfig(block_size=block, num_blocks=max(batches) * -(-max_len // block),
+                                                   max_num_seqs=max(batches), max_num_batched_tokens=max(2048, T),
+                                                   max_model_len=max_len, enable_prefix_caching=False), seed=0)  # fmt: skip
+        engine.warm_up()
+        one = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
+        for i in range(2):
+            engine.generate([prompt(99 - i, T, vocab)], one)
+        times = []
+        for i in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            engine.generate([prompt(90 + i, T, vocab)], one)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        out = {"weights_GB": round(model.num_weight_bytes / 1e9, 2), "prefill_tokens": T,
+               "prefill_ms": round(sorted(times)[1] * 1e3, 3), "prefill_tok_s": round(T / sorted(times)[1], 1)}  # fmt: skip
+        for batch in batches:
+            handles = [engine.submit(prompt(b, context, vocab), greedy) for b in range(batch)]
+            while engine.scheduler.waiting or not engine.scheduler.running or any(
+                    s.num_computed_tokens < s.num_prompt_tokens for s in engine.scheduler.running):  # fmt: skip
+                engine.step()
+            for _ in range(args.warmup):
+                engine.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                engine.step()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            for h in handles:
+                engine.abort(h.id)
+            engine.step()
+            out[f"decode_b{batch}_tok_s"] = round(batch * steps / dt, 1)
+            out[f"decode_b{batch}_ms"] = round(dt / steps * 1e3, 4)
+        del engine, model
+        torch.cuda.empty_cache()
+        return out
+
+    sizes = {}
+    for width in [int(w) for w in args.widths.split(",") if w]:
+        heads = width // 128
+        qwen = Qwen3Config(vocab_size=vocab, hidden_size=width, intermediate_size=3 * width, num_layers=layers,
+                           num_heads=heads, num_kv_heads=max(1, heads // 4), head_dim=128, rms_norm_eps=1e-6,
+                           rope_theta=1e6, tie_word_embeddings=False, max_position_embeddings=40960)  # fmt: skip
+        sizes[str(width)] = {"dozusun": measure(dozusun_config(width, layers, vocab)), "qwen3": measure(qwen)}
+        print(f"width {width}: {json.dumps(sizes[str(width)])}", file=sys.stderr, flush=True)
+    widest = sizes[max(sizes, key=int)]
+    return {
+        "metric": f"decode tok/s at batch {args.batch}, {context}-token contexts (Dozusun layers of width {max(sizes, key=int)}, random weights)",
+        "value": widest["dozusun"][f"decode_b{args.batch}_tok_s"],
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": widest["dozusun"][f"decode_b{args.batch}_ms"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.dtype, "data": "synthetic token ids, random-init weights",
+        "config": {"model": "Dozusun layers beside Qwen3 layers of equal size", "layers": layers, "vocab": vocab,
+                   "global_batch": args.batch, "seq_len": context, "block_size": block, "parallelism": "single GPU",
+                   "sampling": "greedy"},
+        "sizes": sizes,
+    }  # fmt: skip
+
+
 def calibrate(device) -> dict:
     """What this GPU delivers to plain library calls, to read the roofline fractions against: a
     1 GiB device copy (bytes read plus written per second) and an 8192^3 bf16 matrix product."""
@@ -194,6 +305,9 @@ def main() -> int:
     from atomserve_amd.weights.loader import DictSource, bind_checkpoint
     from atomserve_amd.weights.random_init import random_checkpoint
 
+    if args.design == "dozusun":
+        print(json.dumps(design_comparison(args)))
+        return 0
     device = "cuda:0"
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     calibration = None if args.no_calibration else calibrate(device)
