@@ -570,7 +570,10 @@ extern "C" int as_rmsnorm_multi(float* x, const void* d1, const void* d2, const 
                                 int num_out_rows, int n, int update_x, hipStream_t stream) {
   if (num_out_rows <= 0) return AS_OK;
   if (n <= 0 || !out1 || !w1 || (out2 && !w2)) return AS_BAD_SHAPE;
-  const int threads = n >= 2048 ? 256 : (n >= 512 ? 128 : 64);
+  // few rows (a decode step): two columns a thread, every load of a row in flight at once; many rows: fuller threads
+  int threads = num_out_rows >= 512 ? (n + 7) / 8 : (n + 1) / 2;
+  threads = ((threads + 63) / 64) * 64;
+  if (threads > 1024) threads = 1024;
 #define LAUNCH(O, W)                                                                                        \
   rmsnorm_multi_kernel<O, W><<<num_out_rows, threads, 0, stream>>>(x, (const O*)d1, (const O*)d2, rows,     \
                                                                    (const W*)w1, (const W*)w2, eps, (O*)out1, \

@@ -147,9 +147,11 @@ extern "C" int as_delta_prepare(float* qkv, int C, int G, int dim, int H, const 
 // registers for all the row's tokens: lane = slice * CJ + column, a slice being RPL rows of S
 // (64 / CJ slices cover dim).  With p = S_old^T k and r = S_old^T q, both taken in one pass over the
 // old state:  u = beta (v - g p),  S_new = g S_old + k u^T,  o = g r + u (k . q).
-// Keys and queries of TB tokens at a time go through LDS (one round of loads per TB tokens, not one
-// per token).
+// Keys and queries of DELTA_TB tokens at a time go through LDS: a round's loads (16 bytes a lane, all asked
+// for together, with the lanes' own values, betas and decays) are in flight while the round before is
+// worked on, so the chain of dependent steps is the arithmetic alone.  Needs dim % 4 == 0.
 #define DELTA_TB 8
+#define DELTA_STAGE 8  // 16-byte pieces a lane brings per pass of a round's staging
 template <int RPL>
 __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ qkv, int C, int G, int dim, int H,
                                                         int vdim, int CJ, const float* __restrict__ beta,
@@ -174,14 +176,24 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
 #pragma unroll
   for (int i = 0; i < RPL; ++i) S[i] = (carried && live && i0 + i < dim) ? mine[(size_t)(i0 + i) * vdim + j] : 0.f;
   const int q_col = g * dim, k_col = (G + g) * dim, v_col = 2 * G * dim + h * vdim;
-  for (int t0 = 0; t0 < len; t0 += DELTA_TB) {
+  // a round's keys and queries as 16-byte pieces: piece -> (token, key or query, four coordinates)
+  const int quads = dimp >> 2, per_token = 2 * quads, pieces = DELTA_TB * per_token;
+  const int passes = (pieces + WAVE * DELTA_STAGE - 1) / (WAVE * DELTA_STAGE);
+  float4 stage[DELTA_STAGE];
+  float vj[DELTA_TB], bt[DELTA_TB], gt[DELTA_TB];
+  auto fetch = [&](int t0, int pass) {
     const int nt = min(DELTA_TB, len - t0);
-    __syncthreads();
-    for (int e = lane; e < nt * 2 * dimp; e += WAVE) {
-      const int tt = e / (2 * dimp), rest = e % (2 * dimp), which = rest / dimp, i = rest % dimp;
-      lds[e] = i < dim ? qkv[(size_t)(first + t0 + tt) * C + (which ? q_col : k_col) + i] : 0.f;
+#pragma unroll
+    for (int u = 0; u < DELTA_STAGE; ++u) {
+      const int piece = (pass * DELTA_STAGE + u) * WAVE + lane;
+      const int tt = piece / per_token, rest = piece - tt * per_token, which = rest >= quads, i = (rest - which * quads) * 4;
+      stage[u] = (tt < nt && i < dim && piece < pieces)
+                     ? *reinterpret_cast<const float4*>(qkv + (size_t)(first + t0 + tt) * C + (which ? q_col : k_col) + i)
+                     : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    float vj[DELTA_TB], bt[DELTA_TB], gt[DELTA_TB];
+  };
+  auto fetch_own = [&](int t0) {
+    const int nt = min(DELTA_TB, len - t0);
 #pragma unroll
     for (int tt = 0; tt < DELTA_TB; ++tt) {
       const size_t t = (size_t)first + t0 + (tt < nt ? tt : 0);
@@ -189,7 +201,34 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
       bt[tt] = beta[t * H + h];
       gt[tt] = decay[t * H + h];
     }
+  };
+  auto put = [&](int pass) {
+#pragma unroll
+    for (int u = 0; u < DELTA_STAGE; ++u) {
+      const int piece = (pass * DELTA_STAGE + u) * WAVE + lane;
+      if (piece < pieces) *reinterpret_cast<float4*>(lds + (size_t)piece * 4) = stage[u];
+    }
+  };
+  if (len > 0) {
+    fetch(0, 0);
+    fetch_own(0);
+  }
+  for (int t0 = 0; t0 < len; t0 += DELTA_TB) {
+    const int nt = min(DELTA_TB, len - t0);
+    __syncthreads();  // the round before has been read
+    put(0);
+    for (int pass = 1; pass < passes; ++pass) {  // heads wider than a pass brings: the rest, pass by pass
+      fetch(t0, pass);
+      put(pass);
+    }
+    float v_now[DELTA_TB], b_now[DELTA_TB], g_now[DELTA_TB];
+#pragma unroll
+    for (int tt = 0; tt < DELTA_TB; ++tt) { v_now[tt] = vj[tt]; b_now[tt] = bt[tt]; g_now[tt] = gt[tt]; }
     __syncthreads();
+    if (t0 + DELTA_TB < len) {  // in flight while this round is worked on
+      fetch(t0 + DELTA_TB, 0);
+      fetch_own(t0 + DELTA_TB);
+    }
 #pragma unroll
     for (int tt = 0; tt < DELTA_TB; ++tt) {
       if (tt < nt) {
@@ -207,8 +246,8 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
           rr += __shfl_xor(rr, off, WAVE);
           kq += __shfl_xor(kq, off, WAVE);
         }
-        const float gg = gt[tt];
-        const float u = bt[tt] * (vj[tt] - gg * p);
+        const float gg = g_now[tt];
+        const float u = b_now[tt] * (v_now[tt] - gg * p);
 #pragma unroll
         for (int i = 0; i < RPL; ++i) S[i] = fmaf(kk[i], u, gg * S[i]);
         if (live && slice == 0) out[((size_t)(first + t0 + tt) * H + h) * vdim + j] = fmaf(gg, rr, u * kq);
@@ -227,13 +266,14 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
                              const int* row_start, const int* row_slots, int writes, float* out, int num_rows,
                              hipStream_t stream) {
   if (num_rows <= 0) return AS_OK;
-  if (G <= 0 || H <= 0 || H % G || dim <= 0 || vdim <= 0 || dim > 64 * 64 || C < 2 * G * dim + H * vdim || H > 65535)
+  if (G <= 0 || H <= 0 || H % G || dim <= 0 || (dim & 3) || (C & 3) || vdim <= 0 || dim > 64 * 64 ||
+      C < 2 * G * dim + H * vdim || H > 65535)
     return AS_BAD_SHAPE;
   int slices = 1;
   while ((dim + slices - 1) / slices > 64) slices *= 2;  // a lane keeps at most 64 rows of its column
   // few rows and heads: narrower column groups (more slices of fewer rows) until the waves fill the GPU
   while (slices < 8 && (dim + 2 * slices - 1) / (2 * slices) >= 8 &&
-         (long)num_rows * H * ((vdim + WAVE / slices - 1) / (WAVE / slices)) < 4L * compute_units())
+         (long)num_rows * H * ((vdim + WAVE / slices - 1) / (WAVE / slices)) < 8L * compute_units())
     slices *= 2;
   const int rows_per_lane = (dim + slices - 1) / slices;
   const int RPL = rows_per_lane <= 8 ? 8 : rows_per_lane <= 16 ? 16 : rows_per_lane <= 32 ? 32 : 64;
@@ -348,12 +388,67 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restric
   }
 }
 
+// The same for a few tokens (a decode step): the two matrices are streamed once, a wave per output
+// channel, its lanes sharing the inputs (four to a lane per pass, sums over the lanes in a fixed order);
+// four tokens at a time.
+template <typename W>
+__global__ __launch_bounds__(256) void rglru_gates_few_kernel(const float* __restrict__ u, int width, int bw,
+                                                              const W* __restrict__ ra, const W* __restrict__ ra_b,
+                                                              const W* __restrict__ ri, const W* __restrict__ ri_b,
+                                                              const W* __restrict__ lam, float c,
+                                                              float* __restrict__ a_out, float* __restrict__ x_out,
+                                                              int num_tokens) {
+  const int lane = threadIdx.x & (WAVE - 1), ch = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (ch >= width) return;
+  const int b = ch / bw, o = ch - b * bw;
+  const W* wr = ra + ((size_t)b * bw + o) * bw;
+  const W* wi = ri + ((size_t)b * bw + o) * bw;
+  const float rb = to_f32(ra_b[ch]), ib = to_f32(ri_b[ch]), sp = softplusf_(to_f32(lam[ch]));
+  for (int t0 = 0; t0 < num_tokens; t0 += 4) {
+    float accr[4] = {0.f, 0.f, 0.f, 0.f}, acci[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = lane; k < bw; k += WAVE) {
+      const float a = to_f32(wr[k]), bb = to_f32(wi[k]);
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {
+        const float uu = t0 + tt < num_tokens ? u[(size_t)(t0 + tt) * width + b * bw + k] : 0.f;
+        accr[tt] = fmaf(a, uu, accr[tt]);
+        acci[tt] = fmaf(bb, uu, acci[tt]);
+      }
+    }
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+      const float sr = wave_sum(accr[tt]), si = wave_sum(acci[tt]);
+      const int t = t0 + tt;
+      if (lane == 0 && t < num_tokens) {
+        const float rg = sigmoidf_(sr + rb), ig = sigmoidf_(si + ib);
+        const float log_a = -c * rg * sp;
+        a_out[(size_t)t * width + ch] = expf(log_a);
+        x_out[(size_t)t * width + ch] = sqrtf(-expm1f(2.0f * log_a)) * ig * u[(size_t)t * width + ch];
+      }
+    }
+  }
+}
+
+#define GATE_FEW_TOKENS 16
 extern "C" int as_rglru_gates(const float* u, int width, int blocks, const void* ra, const void* ra_b, const void* ri,
                               const void* ri_b, const void* lam, int w_dtype, float c, float* a_out, float* x_out,
                               int num_tokens, hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
   if (width <= 0 || blocks <= 0 || width % blocks || blocks > 65535) return AS_BAD_SHAPE;
   const int bw = width / blocks;
+  if (num_tokens <= GATE_FEW_TOKENS) {
+    const int blocks_few = (width + 3) / 4;
+    if (w_dtype == DT_F32)
+      rglru_gates_few_kernel<float><<<blocks_few, 256, 0, stream>>>(u, width, bw, (const float*)ra, (const float*)ra_b,
+                                                                   (const float*)ri, (const float*)ri_b,
+                                                                   (const float*)lam, c, a_out, x_out, num_tokens);
+    else if (w_dtype == DT_BF16)
+      rglru_gates_few_kernel<bf16><<<blocks_few, 256, 0, stream>>>(u, width, bw, (const bf16*)ra, (const bf16*)ra_b,
+                                                                  (const bf16*)ri, (const bf16*)ri_b, (const bf16*)lam,
+                                                                  c, a_out, x_out, num_tokens);
+    else return AS_BAD_DTYPE;
+    return launch_status();
+  }
   dim3 grid((num_tokens + GATE_TT - 1) / GATE_TT, blocks, (bw + GATE_TO - 1) / GATE_TO);
   if (grid.z > 65535) return AS_BAD_SHAPE;
   if (w_dtype == DT_F32)
