@@ -144,27 +144,41 @@ extern "C" int as_delta_prepare(float* qkv, int C, int G, int dim, int H, const 
 // The scan.  Per head the state S [dim, vdim] moves on token by token:
 //   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q     (o sees the token's own write)
 // The columns of S never meet, so a wave owns CJ columns of one head of one row and keeps them in
-// registers for all the row's tokens: lane = slice * CJ + column, a slice being RPL rows of S
-// (64 / CJ slices cover dim).  With p = S_old^T k and r = S_old^T q, both taken in one pass over the
+// registers for all the row's tokens: lane = column * SL + slice, a slice being RPL rows of S
+// (SL = 64 / CJ slices cover dim; the slices of a column are neighbouring lanes, whose partial sums
+// meet through DPP moves within a row of 16 lanes, not through LDS).  With p = S_old^T k and r = S_old^T q, both taken in one pass over the
 // old state:  u = beta (v - g p),  S_new = g S_old + k u^T,  o = g r + u (k . q).
 // Keys and queries of DELTA_TB tokens at a time go through LDS: a round's loads (16 bytes a lane, all asked
 // for together, with the lanes' own values, betas and decays) are in flight while the round before is
 // worked on, so the chain of dependent steps is the arithmetic alone.  Needs dim % 4 == 0.
 #define DELTA_TB 8
 #define DELTA_STAGE 8  // 16-byte pieces a lane brings per pass of a round's staging
-template <int RPL>
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+// The sum over SL neighbouring lanes (SL = 1, 2, 4, 8), in every one of them: lane ^ 1, lane ^ 2, then
+// the mirror image within eight lanes (which lies in the other four).
+template <int SL> __device__ __forceinline__ float slices_sum(float v) {
+  if (SL >= 2) v += dpp_move<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  if (SL >= 4) v += dpp_move<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  if (SL >= 8) v += dpp_move<0x141>(v);  // row_half_mirror
+  return v;
+}
+
+template <int RPL, int SL>
 __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ qkv, int C, int G, int dim, int H,
-                                                        int vdim, int CJ, const float* __restrict__ beta,
+                                                        int vdim, const float* __restrict__ beta,
                                                         const float* __restrict__ decay, float* __restrict__ state,
                                                         const int* __restrict__ row_first,
                                                         const int* __restrict__ row_len,
                                                         const int* __restrict__ row_start,
                                                         const int* __restrict__ row_slots, int writes,
                                                         float* __restrict__ out) {
-  extern __shared__ float lds[];  // [DELTA_TB][2][dimp]: key then query of each token, dimp = slices * RPL
+  extern __shared__ __attribute__((aligned(16))) float lds[];  // [DELTA_TB][2][dimp]: key then query of each token, dimp = SL * RPL
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int col = lane % CJ, slice = lane / CJ, slices = WAVE / CJ;
-  const int dimp = slices * RPL;
+  constexpr int CJ = WAVE / SL;
+  const int col = lane / SL, slice = lane % SL;
+  constexpr int dimp = SL * RPL;
   const int j = blockIdx.z * CJ + col;
   const bool live = j < vdim;
   const int g = h / (H / G);
@@ -232,20 +246,29 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
 #pragma unroll
     for (int tt = 0; tt < DELTA_TB; ++tt) {
       if (tt < nt) {
-        const float* kk = lds + (size_t)tt * 2 * dimp + i0;
-        const float* qq = kk + dimp;
-        float p = 0.f, rr = 0.f, kq = 0.f;
+        // this lane's slice of the token's key and query, 16 bytes at a time (i0 is a multiple of 8)
+        const float4* k4 = reinterpret_cast<const float4*>(lds + tt * 2 * dimp + i0);
+        const float4* q4 = reinterpret_cast<const float4*>(lds + tt * 2 * dimp + dimp + i0);
+        float kk[RPL], qq[RPL];
 #pragma unroll
-        for (int i = 0; i < RPL; ++i) {
+        for (int i = 0; i < RPL / 4; ++i) {
+          const float4 a = k4[i], b = q4[i];
+          kk[4 * i] = a.x; kk[4 * i + 1] = a.y; kk[4 * i + 2] = a.z; kk[4 * i + 3] = a.w;
+          qq[4 * i] = b.x; qq[4 * i + 1] = b.y; qq[4 * i + 2] = b.z; qq[4 * i + 3] = b.w;
+        }
+        float p = 0.f, rr = 0.f, kq = 0.f, p2 = 0.f, rr2 = 0.f, kq2 = 0.f;  // two chains each: half the dependent steps
+#pragma unroll
+        for (int i = 0; i < RPL; i += 2) {
           p = fmaf(S[i], kk[i], p);
           rr = fmaf(S[i], qq[i], rr);
           kq = fmaf(kk[i], qq[i], kq);
+          p2 = fmaf(S[i + 1], kk[i + 1], p2);
+          rr2 = fmaf(S[i + 1], qq[i + 1], rr2);
+          kq2 = fmaf(kk[i + 1], qq[i + 1], kq2);
         }
-        for (int off = CJ; off < WAVE; off <<= 1) {
-          p += __shfl_xor(p, off, WAVE);
-          rr += __shfl_xor(rr, off, WAVE);
-          kq += __shfl_xor(kq, off, WAVE);
-        }
+        p = slices_sum<SL>(p + p2);
+        rr = slices_sum<SL>(rr + rr2);
+        kq = slices_sum<SL>(kq + kq2);
         const float gg = g_now[tt];
         const float u = b_now[tt] * (v_now[tt] - gg * p);
 #pragma unroll
@@ -269,6 +292,7 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
   if (G <= 0 || H <= 0 || H % G || dim <= 0 || (dim & 3) || (C & 3) || vdim <= 0 || dim > 64 * 64 ||
       C < 2 * G * dim + H * vdim || H > 65535)
     return AS_BAD_SHAPE;
+  if (dim > 8 * 64) return AS_BAD_SHAPE;  // eight slices of 64 rows
   int slices = 1;
   while ((dim + slices - 1) / slices > 64) slices *= 2;  // a lane keeps at most 64 rows of its column
   // few rows and heads: narrower column groups (more slices of fewer rows) until the waves fill the GPU
@@ -280,13 +304,21 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
   const int CJ = WAVE / slices;
   dim3 grid(num_rows, H, (vdim + CJ - 1) / CJ);
   const size_t lds = (size_t)DELTA_TB * 2 * slices * RPL * sizeof(float);
-#define LAUNCH(R)                                                                                              \
-  delta_scan_kernel<R><<<grid, 64, lds, stream>>>(qkv, C, G, dim, H, vdim, CJ, beta, decay, state, row_first,  \
-                                                  row_len, row_start, row_slots, writes, out)
-  if (RPL == 8) LAUNCH(8);
-  else if (RPL == 16) LAUNCH(16);
-  else if (RPL == 32) LAUNCH(32);
-  else LAUNCH(64);
+#define LAUNCH(R, SLV)                                                                                          \
+  delta_scan_kernel<R, SLV><<<grid, 64, lds, stream>>>(qkv, C, G, dim, H, vdim, beta, decay, state, row_first,  \
+                                                       row_len, row_start, row_slots, writes, out)
+#define LAUNCH_SL(R)              \
+  do {                            \
+    if (slices == 1) LAUNCH(R, 1);      \
+    else if (slices == 2) LAUNCH(R, 2); \
+    else if (slices == 4) LAUNCH(R, 4); \
+    else LAUNCH(R, 8);                  \
+  } while (0)
+  if (RPL == 8) LAUNCH_SL(8);
+  else if (RPL == 16) LAUNCH_SL(16);
+  else if (RPL == 32) LAUNCH_SL(32);
+  else LAUNCH_SL(64);
+#undef LAUNCH_SL
 #undef LAUNCH
   return launch_status();
 }
