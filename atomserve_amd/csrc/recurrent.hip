@@ -156,12 +156,13 @@ extern "C" int as_delta_prepare(float* qkv, int C, int G, int dim, int H, const 
 template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
 }
-// The sum over SL neighbouring lanes (SL = 1, 2, 4, 8), in every one of them: lane ^ 1, lane ^ 2, then
-// the mirror image within eight lanes (which lies in the other four).
+// The sum over SL neighbouring lanes (SL = 1, 2, 4, 8, 16), in every one of them: lane ^ 1, lane ^ 2, then
+// the mirror image within eight lanes (which lies in the other four) and within sixteen (the other eight).
 template <int SL> __device__ __forceinline__ float slices_sum(float v) {
   if (SL >= 2) v += dpp_move<0xB1>(v);   // quad_perm [1, 0, 3, 2]
   if (SL >= 4) v += dpp_move<0x4E>(v);   // quad_perm [2, 3, 0, 1]
   if (SL >= 8) v += dpp_move<0x141>(v);  // row_half_mirror
+  if (SL >= 16) v += dpp_move<0x140>(v);  // row_mirror
   return v;
 }
 
@@ -292,11 +293,11 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
   if (G <= 0 || H <= 0 || H % G || dim <= 0 || (dim & 3) || (C & 3) || vdim <= 0 || dim > 64 * 64 ||
       C < 2 * G * dim + H * vdim || H > 65535)
     return AS_BAD_SHAPE;
-  if (dim > 8 * 64) return AS_BAD_SHAPE;  // eight slices of 64 rows
+  if (dim > 16 * 64) return AS_BAD_SHAPE;  // sixteen slices of 64 rows
   int slices = 1;
   while ((dim + slices - 1) / slices > 64) slices *= 2;  // a lane keeps at most 64 rows of its column
   // few rows and heads: narrower column groups (more slices of fewer rows) until the waves fill the GPU
-  while (slices < 8 && (dim + 2 * slices - 1) / (2 * slices) >= 8 &&
+  while (slices < 16 && (dim + 2 * slices - 1) / (2 * slices) >= 8 &&
          (long)num_rows * H * ((vdim + WAVE / slices - 1) / (WAVE / slices)) < 8L * compute_units())
     slices *= 2;
   const int rows_per_lane = (dim + slices - 1) / slices;
@@ -312,7 +313,8 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
     if (slices == 1) LAUNCH(R, 1);      \
     else if (slices == 2) LAUNCH(R, 2); \
     else if (slices == 4) LAUNCH(R, 4); \
-    else LAUNCH(R, 8);                  \
+    else if (slices == 8) LAUNCH(R, 8); \
+    else LAUNCH(R, 16);                 \
   } while (0)
   if (RPL == 8) LAUNCH_SL(8);
   else if (RPL == 16) LAUNCH_SL(16);
