@@ -83,66 +83,81 @@ extern "C" int as_moe_route_table(const int* token_ids, const int* table, int vo
 //
 // bf16: v_mfma_f32_16x16x32_bf16 with the weights as the A operand (16 rows of w) and 16 of the tile's
 // pairs as the B operand.  A wave owns 16 outputs (and their up rows) for all of the tile's pairs (up to
-// four column tiles of 16); the tile's activations are brought into LDS once per round of 128 inputs for
-// the four waves (rows padded by 16 bytes against bank conflicts), the weights go from memory straight
-// into registers, 16 bytes a lane.  Few pairs (a decode step) cost few products: column tiles beyond the
-// tile's count are skipped.  Needs K % 8 == 0.
+// four column tiles of 16).  Per round of 128 inputs the workgroup brings the tile's activations and its 64
+// (gated: 128) weight rows into LDS, whole 256-byte runs of a row per 16 lanes, rows padded by 16 bytes
+// against bank conflicts; the next round's loads are in flight while this round is multiplied.  Few pairs
+// (a decode step) cost few products: column tiles beyond the tile's count are skipped.  Needs K % 8 == 0.
 template <bool GATED, typename OutT>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restrict__ a, int a_div,
                                                             const bf16* __restrict__ w, int N, int K,
                                                             const int* __restrict__ order,
                                                             const int* __restrict__ tiles,
                                                             const int* __restrict__ counts, OutT* __restrict__ out) {
+  constexpr int WROWS = GATED ? 2 * MOE_STRIP : MOE_STRIP;  // weight rows of a round: the strip's, then their up rows
+  constexpr int WLOADS = WROWS * (MOE_KC / 8) / 256;        // 16-byte pieces of them per thread
   __shared__ __attribute__((aligned(16))) bf16 acts[MOE_TILE][MOE_KC + 8];
+  __shared__ __attribute__((aligned(16))) bf16 wts[WROWS][MOE_KC + 8];
   __shared__ int pair_of[MOE_TILE];
   const int tile = blockIdx.y;
   if (tile >= counts[0]) return;
   const int e = tiles[3 * tile], at = tiles[3 * tile + 1], cnt = tiles[3 * tile + 2];
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
   const int lr = lane & 15, lg = lane >> 4;
-  const int n0 = blockIdx.x * MOE_STRIP + wave * 16;
+  const int nb = blockIdx.x * MOE_STRIP, n0 = nb + wave * 16;
   const int col_tiles = (cnt + 15) >> 4;
   if (threadIdx.x < MOE_TILE) pair_of[threadIdx.x] = threadIdx.x < cnt ? order[at + threadIdx.x] : -1;
   __syncthreads();
   const int NW = GATED ? 2 * N : N;
   const bf16* wbase = w + (size_t)e * NW * K;
-  const bool row_in = n0 + lr < N;
-  const bf16* wrow = wbase + (size_t)(row_in ? n0 + lr : 0) * K;
-  const bf16* urow = wbase + (size_t)(N + (row_in ? n0 + lr : 0)) * K;
   floatx4 acc[4], acc_up[4];
 #pragma unroll
   for (int ct = 0; ct < 4; ++ct) { acc[ct] = floatx4{0.f, 0.f, 0.f, 0.f}; acc_up[ct] = floatx4{0.f, 0.f, 0.f, 0.f}; }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  // staging: thread -> (row of the tile, 16-byte piece of the round): 64 rows x 16 pieces, four a thread
+  // thread -> (row, 16-byte piece of the round): 16 pieces a row, so 16 lanes read 256 bytes of a row in a run
+  const int piece_k = (threadIdx.x & 15) * 8, piece_row = threadIdx.x >> 4;  // rows piece_row + 16 i
+  const bf16* arow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = piece_row + 16 * i;
+    const int pair = row < col_tiles * 16 ? pair_of[row] : -1;
+    arow[i] = pair >= 0 ? a + (size_t)(pair / a_div) * K : nullptr;
+  }
+  bf16x8 staged[4], wstaged[WLOADS];
+  auto fetch = [&](int k0) {
+    const bool k_in = k0 + piece_k < K;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      staged[i] = (arow[i] && k_in) ? *reinterpret_cast<const bf16x8*>(arow[i] + k0 + piece_k) : zero;
+#pragma unroll
+    for (int i = 0; i < WLOADS; ++i) {
+      const int row = piece_row + 16 * i;                       // of the round's weight rows
+      const int n = nb + (row & (MOE_STRIP - 1));               // the output it belongs to
+      const size_t wr = (size_t)((GATED && row >= MOE_STRIP) ? N + n : n);
+      wstaged[i] = (n < N && k_in) ? *reinterpret_cast<const bf16x8*>(wbase + wr * K + k0 + piece_k) : zero;
+    }
+  };
+  fetch(0);
   for (int k0 = 0; k0 < K; k0 += MOE_KC) {
-    __syncthreads();
+    __syncthreads();  // the round before has been read
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int piece = threadIdx.x + i * 256, row = piece >> 4, kk = (piece & 15) * 8;
-      if (row < col_tiles * 16) {
-        const int pair = pair_of[row];
-        const bf16x8 v = (pair >= 0 && k0 + kk < K) ? *reinterpret_cast<const bf16x8*>(a + (size_t)(pair / a_div) * K + k0 + kk) : zero;
-        *reinterpret_cast<bf16x8*>(&acts[row][kk]) = v;
-      }
-    }
-    bf16x8 wv[MOE_KC / 32], uv[MOE_KC / 32];
+    for (int i = 0; i < 4; ++i)
+      if (piece_row + 16 * i < col_tiles * 16) *reinterpret_cast<bf16x8*>(&acts[piece_row + 16 * i][piece_k]) = staged[i];
 #pragma unroll
-    for (int s = 0; s < MOE_KC / 32; ++s) {
-      const int k = k0 + s * 32 + lg * 8;
-      const bool in = row_in && k < K;
-      wv[s] = in ? *reinterpret_cast<const bf16x8*>(wrow + k) : zero;
-      if (GATED) uv[s] = in ? *reinterpret_cast<const bf16x8*>(urow + k) : zero;
-    }
+    for (int i = 0; i < WLOADS; ++i) *reinterpret_cast<bf16x8*>(&wts[piece_row + 16 * i][piece_k]) = wstaged[i];
     __syncthreads();
+    if (k0 + MOE_KC < K) fetch(k0 + MOE_KC);  // in flight while this round is multiplied
     if (n0 < N) {
 #pragma unroll
       for (int s = 0; s < MOE_KC / 32; ++s) {
+        const bf16x8 wv = *reinterpret_cast<const bf16x8*>(&wts[wave * 16 + lr][s * 32 + lg * 8]);
+        bf16x8 uv = zero;
+        if (GATED) uv = *reinterpret_cast<const bf16x8*>(&wts[MOE_STRIP + wave * 16 + lr][s * 32 + lg * 8]);
 #pragma unroll
         for (int ct = 0; ct < 4; ++ct) {
           if (ct < col_tiles) {
             const bf16x8 av = *reinterpret_cast<const bf16x8*>(&acts[ct * 16 + lr][s * 32 + lg * 8]);
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[s], av, acc[ct], 0, 0, 0);
-            if (GATED) acc_up[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv[s], av, acc_up[ct], 0, 0, 0);
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc[ct], 0, 0, 0);
+            if (GATED) acc_up[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv, av, acc_up[ct], 0, 0, 0);
           }
         }
       }
