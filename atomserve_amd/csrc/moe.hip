@@ -86,7 +86,17 @@ extern "C" int as_moe_route_table(const int* token_ids, const int* table, int vo
 // four column tiles of 16).  Per round of 128 inputs the workgroup brings the tile's activations and its 64
 // (gated: 128) weight rows into LDS, whole 256-byte runs of a row per 16 lanes, rows padded by 16 bytes
 // against bank conflicts; the next round's loads are in flight while this round is multiplied.  Few pairs
-// (a decode step) cost few products: column tiles beyond the tile's count are skipped.  Needs K % 8 == 0.
+// (a decode step) cost few products: column tiles beyond the tile's count are skipped.  Rows of any width (16-byte loads where K % 8 == 0, single values else).
+// Eight inputs of a row from column k on: 16 bytes at once where rows are multiples of 8 wide (then every
+// row starts on 16 bytes and K ends on a piece's end), else one by one, zeros beyond the row's end.
+__device__ __forceinline__ bf16x8 row_piece(const bf16* row, int k, int K, bool whole) {
+  if (whole) return *reinterpret_cast<const bf16x8*>(row + k);
+  bf16x8 v;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = k + i < K ? row[k + i] : (bf16)0.f;
+  return v;
+}
+
 template <bool GATED, typename OutT>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restrict__ a, int a_div,
                                                             const bf16* __restrict__ w, int N, int K,
@@ -113,6 +123,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restri
 #pragma unroll
   for (int ct = 0; ct < 4; ++ct) { acc[ct] = floatx4{0.f, 0.f, 0.f, 0.f}; acc_up[ct] = floatx4{0.f, 0.f, 0.f, 0.f}; }
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bool whole = (K & 7) == 0;
   // thread -> (row, 16-byte piece of the round): 16 pieces a row, so 16 lanes read 256 bytes of a row in a run
   const int piece_k = (threadIdx.x & 15) * 8, piece_row = threadIdx.x >> 4;  // rows piece_row + 16 i
   const bf16* arow[4];
@@ -127,13 +138,13 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restri
     const bool k_in = k0 + piece_k < K;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      staged[i] = (arow[i] && k_in) ? *reinterpret_cast<const bf16x8*>(arow[i] + k0 + piece_k) : zero;
+      staged[i] = (arow[i] && k_in) ? row_piece(arow[i], k0 + piece_k, K, whole) : zero;
 #pragma unroll
     for (int i = 0; i < WLOADS; ++i) {
       const int row = piece_row + 16 * i;                       // of the round's weight rows
       const int n = nb + (row & (MOE_STRIP - 1));               // the output it belongs to
       const size_t wr = (size_t)((GATED && row >= MOE_STRIP) ? N + n : n);
-      wstaged[i] = (n < N && k_in) ? *reinterpret_cast<const bf16x8*>(wbase + wr * K + k0 + piece_k) : zero;
+      wstaged[i] = (n < N && k_in) ? row_piece(wbase + wr * K, k0 + piece_k, K, whole) : zero;
     }
   };
   fetch(0);
@@ -245,7 +256,6 @@ extern "C" int as_moe_gemm(const void* a, int dtype, int a_div, const void* w, i
     return launch_status();
   }
   if (dtype != DT_BF16) return AS_BAD_DTYPE;
-  if (K & 7) return AS_BAD_SHAPE;
   if (gated) {
     if (out_dtype != DT_BF16) return AS_BAD_DTYPE;
     moe_gemm_bf16_kernel<true, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out);

@@ -150,7 +150,7 @@ extern "C" int as_delta_prepare(float* qkv, int C, int G, int dim, int H, const 
 // old state:  u = beta (v - g p),  S_new = g S_old + k u^T,  o = g r + u (k . q).
 // Keys and queries of DELTA_TB tokens at a time go through LDS: a round's loads (16 bytes a lane, all asked
 // for together, with the lanes' own values, betas and decays) are in flight while the round before is
-// worked on, so the chain of dependent steps is the arithmetic alone.  Needs dim % 4 == 0.
+// worked on, so the chain of dependent steps is the arithmetic alone.
 #define DELTA_TB 8
 #define DELTA_STAGE 8  // 16-byte pieces a lane brings per pass of a round's staging
 template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
@@ -196,15 +196,26 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
   const int passes = (pieces + WAVE * DELTA_STAGE - 1) / (WAVE * DELTA_STAGE);
   float4 stage[DELTA_STAGE];
   float vj[DELTA_TB], bt[DELTA_TB], gt[DELTA_TB];
+  const bool whole = ((dim | C) & 3) == 0;  // every key and query starts on 16 bytes
   auto fetch = [&](int t0, int pass) {
     const int nt = min(DELTA_TB, len - t0);
 #pragma unroll
     for (int u = 0; u < DELTA_STAGE; ++u) {
       const int piece = (pass * DELTA_STAGE + u) * WAVE + lane;
       const int tt = piece / per_token, rest = piece - tt * per_token, which = rest >= quads, i = (rest - which * quads) * 4;
-      stage[u] = (tt < nt && i < dim && piece < pieces)
-                     ? *reinterpret_cast<const float4*>(qkv + (size_t)(first + t0 + tt) * C + (which ? q_col : k_col) + i)
-                     : make_float4(0.f, 0.f, 0.f, 0.f);
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (tt < nt && i < dim && piece < pieces) {
+        const float* src = qkv + (size_t)(first + t0 + tt) * C + (which ? q_col : k_col) + i;
+        if (whole) {
+          v = *reinterpret_cast<const float4*>(src);
+        } else {  // widths that are no multiples of 4: value by value
+          v.x = src[0];
+          if (i + 1 < dim) v.y = src[1];
+          if (i + 2 < dim) v.z = src[2];
+          if (i + 3 < dim) v.w = src[3];
+        }
+      }
+      stage[u] = v;
     }
   };
   auto fetch_own = [&](int t0) {
@@ -290,8 +301,7 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
                              const int* row_start, const int* row_slots, int writes, float* out, int num_rows,
                              hipStream_t stream) {
   if (num_rows <= 0) return AS_OK;
-  if (G <= 0 || H <= 0 || H % G || dim <= 0 || (dim & 3) || (C & 3) || vdim <= 0 || dim > 64 * 64 ||
-      C < 2 * G * dim + H * vdim || H > 65535)
+  if (G <= 0 || H <= 0 || H % G || dim <= 0 || vdim <= 0 || C < 2 * G * dim + H * vdim || H > 65535)
     return AS_BAD_SHAPE;
   if (dim > 16 * 64) return AS_BAD_SHAPE;  // sixteen slices of 64 rows
   int slices = 1;

@@ -69,7 +69,7 @@ def step_reserve_bytes(plan, max_batched_tokens: int, max_num_seqs: int) -> int:
 def build_parser() -> argparse.ArgumentParser:
     p = argparse.ArgumentParser(
         prog="atomserve",
-        description="Run a Qwen3 model folder on one MI355X and generate from token-id prompts.",
+        description="Run a model folder (Qwen3, Dozusun) on one MI355X and generate from token-id prompts.",
         formatter_class=argparse.ArgumentDefaultsHelpFormatter,
     )
     p.add_argument("model", help="local model directory (config.json + *.safetensors); with --random-weights, "

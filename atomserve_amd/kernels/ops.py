@@ -1269,8 +1269,6 @@ def moe_gemm(a, w, route: ExpertRoute, out, gated: bool, per_token: bool) -> Non
     if gated and w.shape[1] % 2:
         raise KernelError("moe_gemm: gate and up rows come in equal numbers")
     _check(out, "out", (a.dtype, F32), (pairs, N))
-    if a.dtype == BF16 and K % 8:
-        raise KernelError("moe_gemm: bf16 rows are read 16 bytes at a time (width % 8 == 0)")
     if gated and out.dtype != a.dtype:
         raise KernelError("moe_gemm: the gated product's result has the inputs' dtype")
     call("as_moe_gemm", _ptr(a), _DT[a.dtype], route.top if per_token else 1, _ptr(w), N, K, int(bool(gated)),

@@ -38,9 +38,6 @@ class DeltaRule(Mixer):
             raise ValueError(f"{s.num_heads} value heads do not divide over {s.num_kv_heads} key heads")
         if not 1 <= s.conv.taps <= ops.CONV_MAX_TAPS:
             raise ValueError(f"a short convolution has 1 to {ops.CONV_MAX_TAPS} taps, not {s.conv.taps}")
-        if s.key_dim % 4 or (s.num_heads * s.value_dim) % 4:
-            raise ValueError(f"the scan reads keys 16 bytes at a time: key_dim {s.key_dim} and heads x value_dim "
-                             f"{s.num_heads * s.value_dim} must be multiples of 4")  # fmt: skip
         qk, v = s.num_kv_heads * s.key_dim, s.num_heads * s.value_dim
         self.channels = 2 * qk + v  # what passes the convolution: q, k, v
         # columns of the input product's result: q, k, v, output gate, beta, step size

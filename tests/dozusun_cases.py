@@ -53,6 +53,23 @@ CASES = {
         ],
         "loop": {"start": 0, "stop": 2, "times": 2},
     },  # fmt: skip
+    # delta layers only (no pages at all), widths that are no multiples of 4 or 8, an odd number of heads
+    "delta_only": {
+        "architecture": "Dozusun", "vocab": 90, "width": 44, "norm": {"eps": 1e-5},
+        "layers": [
+            {"type": "delta", "mixer": _delta(3, 3, 6, 10, 2), "mlp": _moe(12, 4, 2)},
+            {"type": "delta", "mixer": _delta(5, 1, 18, 6, 3), "mlp": {"kind": "dense", "ff": 20}},
+        ],
+        "loop": {"start": 1, "stop": 2, "times": 2},
+    },  # fmt: skip
+    # side-by-side layers only, more query heads to a kv head than a matrix tile holds rows for (17), one block a channel
+    "side_only": {
+        "architecture": "Dozusun", "vocab": 64, "width": 48, "norm": {"eps": 1e-6},
+        "layers": [
+            {"type": "parallel", "mixer": _side(17, 1, 8, 4, 0.35, 5, 24, 24, 2, 0.9, 1.1), "mlp": _moe(8, 2, 1)},
+            {"type": "parallel", "mixer": _side(2, 2, 12, 20, 0.3, 33, 40, 2, 3, 1.0, 1.0), "mlp": None},
+        ],
+    },  # fmt: skip
 }
 
 

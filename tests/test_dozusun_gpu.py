@@ -469,3 +469,24 @@ def test_models_of_these_shapes_say_they_replay():
     """Every part is made of launches on the step's device arrays alone, so decode steps are captured."""
     raw = CASES["looped"]
     assert build_model(raw, random_weights(raw, seed=1), "bfloat16").capturable
+
+
+def test_the_command_line_generates_from_a_folder(tmp_path, capsys):
+    """`atomserve FOLDER --prompt-ids ...` on a Dozusun folder written here: the architecture is found by its name
+    in config.json, the weights by their names, and the greedy tokens are the plain model's."""
+    import json
+
+    from safetensors.torch import save_file
+
+    from atomserve_amd.engine import cli
+
+    raw = CASES["all_looped"]
+    weights = random_weights(raw, seed=17)
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    save_file({k: (v if v.dtype == torch.int32 else v.bfloat16()).contiguous() for k, v in weights.items()}, str(tmp_path / "model.safetensors"))
+    prompt = rc.random_ids(raw["vocab"], 21, 3)
+    code = cli.main([str(tmp_path), "--dtype", "fp32", "--prompt-ids", " ".join(map(str, prompt)), "--max-tokens", "5", "--temperature", "0",
+                     "--ignore-eos", "--kv-mem-gb", "0.05", "--max-num-seqs", "2", "--max-batched-tokens", "16"])
+    assert code == 0
+    lines = [json.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
+    assert lines[-1]["output_ids"] == plain.greedy(raw, weights, prompt, 5)
