@@ -70,6 +70,29 @@ __global__ void conv_history_kernel(const T* __restrict__ in, int ld, int col0, 
   for (int h = 0; h < keep; ++h) mine[(size_t)h * C + c] = fresh[h];
 }
 
+// A decode step (every row one token: token t is row t): the convolution and the history's move in one
+// kernel.  A thread owns a channel of a row, so it reads the old inputs before it writes the new ones.
+template <typename T, typename W>
+__global__ void short_conv_step_kernel(const T* __restrict__ in, int ld, int col0, int C, const W* __restrict__ in_bias,
+                                       const W* __restrict__ w, const W* __restrict__ bias, int taps, int act,
+                                       float* __restrict__ history, const int* __restrict__ row_start,
+                                       const int* __restrict__ row_slots, int writes, float* __restrict__ out) {
+  const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int keep = taps - 1, slot = row_slots[t];
+  const bool carried = row_start[t] > 0 && slot >= 0;
+  float* mine = history + (size_t)(slot < 0 ? 0 : slot) * keep * C;
+  float seen[CONV_MAX_TAPS];
+  for (int i = 0; i < keep; ++i) seen[i] = carried ? mine[(size_t)i * C + c] : 0.f;
+  seen[keep] = to_f32(in[(size_t)t * ld + col0 + c]) + (in_bias ? to_f32(in_bias[c]) : 0.f);
+  float acc = 0.f;
+  for (int i = 0; i < taps; ++i) acc = fmaf(to_f32(w[(size_t)c * taps + i]), seen[i], acc);
+  if (bias) acc += to_f32(bias[c]);
+  out[(size_t)t * C + c] = act == 1 ? siluf_(acc) : acc;
+  if (writes && slot >= 0)
+    for (int i = 0; i < keep; ++i) mine[(size_t)i * C + c] = seen[i + 1];
+}
+
 extern "C" int as_short_conv(const void* in, int dtype, int ld, int col0, int C, const void* in_bias, const void* w,
                              const void* bias, int w_dtype, int taps, int act, float* history, const int* tok_row,
                              const int* row_first, const int* row_len, const int* row_start, const int* row_slots,
@@ -81,6 +104,12 @@ extern "C" int as_short_conv(const void* in, int dtype, int ld, int col0, int C,
   if (grid.y > 65535) return AS_BAD_SHAPE;
 #define LAUNCH(T, W)                                                                                              \
   do {                                                                                                            \
+    if (!tok_row && num_rows == num_tokens) { /* every row one token */                                           \
+      short_conv_step_kernel<T, W><<<grid, threads, 0, stream>>>((const T*)in, ld, col0, C, (const W*)in_bias,   \
+                                                                 (const W*)w, (const W*)bias, taps, act, history, \
+                                                                 row_start, row_slots, writes, out);             \
+      break;                                                                                                      \
+    }                                                                                                             \
     short_conv_kernel<T, W><<<grid, threads, 0, stream>>>((const T*)in, ld, col0, C, (const W*)in_bias,          \
                                                           (const W*)w, (const W*)bias, taps, act, history,       \
                                                           tok_row, row_first, row_start, row_slots, out);        \

@@ -20,7 +20,9 @@ from atomserve_amd.parts.base import Mixer, PagedCacheRequest, StateCacheRequest
 
 
 def _step_rows(step):
-    return (step.tok_row, step.row_first, step.row_len, step.row_start, step.row_slots)
+    """(tok_row, row_first, row_len, row_start, row_slots) of a step; tok_row None in a decode step, where token t is
+    row t (the kernels then take the shorter way of rows of one token)."""
+    return (None if step.decode_only else step.tok_row, step.row_first, step.row_len, step.row_start, step.row_slots)
 
 
 class DeltaRule(Mixer):

@@ -378,6 +378,36 @@ def test_a_window_edge_shows(window, block_size):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_without_a_window_finds_a_far_key_among_hundreds(dtype):
+    """No window: the fourth token's key is what the last tokens look for, 330 tokens and 20 pages later; a page
+    lost or a table entry wrong on the way shows at the output's own size.  Met at the end of a long prompt, in a
+    portion behind a long cached prefix and token by token."""
+    a = {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 2.0}
+    r = {"width": 16, "blocks": 2, "conv": 2}
+    hidden, T, mark = 32, 335, 3
+    gen = torch.Generator().manual_seed(77)
+    w = side_weights(hidden, a, r, gen)
+    half = bf(torch.randn(a["dim"], hidden // 2, generator=gen) * 0.5)
+    w["left.q"] = torch.cat([torch.cat([half, torch.zeros_like(half)], dim=1)] * a["heads"])
+    w["left.k"] = torch.cat([torch.cat([torch.zeros_like(half), half], dim=1)] * a["kv_heads"])
+    h = bf(torch.randn(T, hidden, generator=gen) * 0.3)
+    pattern = bf(torch.randn(hidden // 2, generator=gen))
+    h[T - 12 :, : hidden // 2] = pattern
+    h[mark, hidden // 2 :] = pattern
+    h[mark] = h[mark] * 2
+    m = {"left": a, "right": r, "left_scale": 1.0, "right_scale": 0.0}
+    wd = {"x." + k: v.double() for k, v in w.items()}
+    ref = plain.side_by_side_mixer(h.double(), wd, "x.", m, 1e-5).float()
+    without = plain.side_by_side_mixer(h[mark + 1 :].double(), wd, "x.", m, 1e-5).float()
+    assert (without[-1] - ref[-1]).abs().max() > 0.2 * ref[-1].abs().max(), "the far key does not matter in this test"
+    part = bind_side(w, side_spec(hidden, a, r, 1.0, 0.0), dtype)
+    tol = (3e-5 if dtype == "float32" else 4e-2) * max(1.0, float(ref.abs().max()))
+    for cuts in ([T], [T - 12, 12], [T - 12] + [1] * 12, [64, 64, 64, 64, 64, 3, 12], [320, 2, 2, 11]):
+        got = run_mixer(part, h, cuts, dtype)
+        assert (got - ref).abs().max() <= tol, f"{cuts}: {float((got - ref).abs().max()):.3e} of {float(ref.abs().max()):.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("experts,top,ff,T", [(5, 2, 24, 70), (3, 3, 8, 5), (9, 1, 40, 33), (2, 1, 16, 1)])
 def test_table_routed_experts_alone(experts, top, ff, T, dtype):
     from atomserve_amd.engine.batch import Row, StepBatch
