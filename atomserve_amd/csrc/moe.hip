@@ -17,6 +17,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes as they are moved, whatever they hold
 
 // ---- routing ------------------------------------------------------------------------------------
 // table [vocab, top] int32: the experts of every token id.  order [P]: the pairs sorted by expert;
@@ -87,10 +88,9 @@ extern "C" int as_moe_route_table(const int* token_ids, const int* table, int vo
 // (gated: 128) weight rows into LDS, whole 256-byte runs of a row per 16 lanes, rows padded by 16 bytes
 // against bank conflicts; the next round's loads are in flight while this round is multiplied.  Few pairs
 // (a decode step) cost few products: column tiles beyond the tile's count are skipped.  Rows of any width (16-byte loads where K % 8 == 0, single values else).
-// Eight inputs of a row from column k on: 16 bytes at once where rows are multiples of 8 wide (then every
-// row starts on 16 bytes and K ends on a piece's end), else one by one, zeros beyond the row's end.
-__device__ __forceinline__ bf16x8 row_piece(const bf16* row, int k, int K, bool whole) {
-  if (whole) return *reinterpret_cast<const bf16x8*>(row + k);
+// Eight inputs of a row from column k on, one by one, zeros beyond the row's end (rows that do not start on
+// 16 bytes, and a round that reaches beyond K).
+__device__ __forceinline__ bf16x8 row_piece(const bf16* row, int k, int K) {
   bf16x8 v;
 #pragma unroll
   for (int i = 0; i < 8; ++i) v[i] = k + i < K ? row[k + i] : (bf16)0.f;
@@ -122,29 +122,38 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restri
   floatx4 acc[4], acc_up[4];
 #pragma unroll
   for (int ct = 0; ct < 4; ++ct) { acc[ct] = floatx4{0.f, 0.f, 0.f, 0.f}; acc_up[ct] = floatx4{0.f, 0.f, 0.f, 0.f}; }
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   const bool whole = (K & 7) == 0;
-  // thread -> (row, 16-byte piece of the round): 16 pieces a row, so 16 lanes read 256 bytes of a row in a run
+  // thread -> (row, 16-byte piece of the round): 16 pieces a row, so 16 lanes read 256 bytes of a row in a run.
+  // Rows that stand for no pair or no output read a row that exists (their products are never stored); only a
+  // round that reaches beyond K, or rows that do not start on 16 bytes, take the careful way.
   const int piece_k = (threadIdx.x & 15) * 8, piece_row = threadIdx.x >> 4;  // rows piece_row + 16 i
   const bf16* arow[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int row = piece_row + 16 * i;
     const int pair = row < col_tiles * 16 ? pair_of[row] : -1;
-    arow[i] = pair >= 0 ? a + (size_t)(pair / a_div) * K : nullptr;
+    arow[i] = a + (size_t)(pair >= 0 ? pair / a_div : 0) * K;
   }
-  bf16x8 staged[4], wstaged[WLOADS];
+  const bf16* wrow[WLOADS];
+#pragma unroll
+  for (int i = 0; i < WLOADS; ++i) {
+    const int row = piece_row + 16 * i;                                        // of the round's weight rows
+    const int n = min(nb + (row & (MOE_STRIP - 1)), N - 1);                    // the output it belongs to
+    wrow[i] = wbase + (size_t)((GATED && row >= MOE_STRIP) ? N + n : n) * K;
+  }
+  u32x4 staged[4], wstaged[WLOADS];
   auto fetch = [&](int k0) {
-    const bool k_in = k0 + piece_k < K;
+    const int k = k0 + piece_k;
+    if (whole && k0 + MOE_KC <= K) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      staged[i] = (arow[i] && k_in) ? row_piece(arow[i], k0 + piece_k, K, whole) : zero;
+      for (int i = 0; i < 4; ++i) staged[i] = *reinterpret_cast<const u32x4*>(arow[i] + k);
 #pragma unroll
-    for (int i = 0; i < WLOADS; ++i) {
-      const int row = piece_row + 16 * i;                       // of the round's weight rows
-      const int n = nb + (row & (MOE_STRIP - 1));               // the output it belongs to
-      const size_t wr = (size_t)((GATED && row >= MOE_STRIP) ? N + n : n);
-      wstaged[i] = (n < N && k_in) ? row_piece(wbase + wr * K, k0 + piece_k, K, whole) : zero;
+      for (int i = 0; i < WLOADS; ++i) wstaged[i] = *reinterpret_cast<const u32x4*>(wrow[i] + k);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) staged[i] = __builtin_bit_cast(u32x4, row_piece(arow[i], k, K));
+#pragma unroll
+      for (int i = 0; i < WLOADS; ++i) wstaged[i] = __builtin_bit_cast(u32x4, row_piece(wrow[i], k, K));
     }
   };
   fetch(0);
@@ -152,16 +161,16 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restri
     __syncthreads();  // the round before has been read
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (piece_row + 16 * i < col_tiles * 16) *reinterpret_cast<bf16x8*>(&acts[piece_row + 16 * i][piece_k]) = staged[i];
+      if (piece_row + 16 * i < col_tiles * 16) *reinterpret_cast<u32x4*>(&acts[piece_row + 16 * i][piece_k]) = staged[i];
 #pragma unroll
-    for (int i = 0; i < WLOADS; ++i) *reinterpret_cast<bf16x8*>(&wts[piece_row + 16 * i][piece_k]) = wstaged[i];
+    for (int i = 0; i < WLOADS; ++i) *reinterpret_cast<u32x4*>(&wts[piece_row + 16 * i][piece_k]) = wstaged[i];
     __syncthreads();
     if (k0 + MOE_KC < K) fetch(k0 + MOE_KC);  // in flight while this round is multiplied
     if (n0 < N) {
 #pragma unroll
       for (int s = 0; s < MOE_KC / 32; ++s) {
         const bf16x8 wv = *reinterpret_cast<const bf16x8*>(&wts[wave * 16 + lr][s * 32 + lg * 8]);
-        bf16x8 uv = zero;
+        bf16x8 uv = wv;
         if (GATED) uv = *reinterpret_cast<const bf16x8*>(&wts[MOE_STRIP + wave * 16 + lr][s * 32 + lg * 8]);
 #pragma unroll
         for (int ct = 0; ct < 4; ++ct) {
