@@ -9,6 +9,7 @@
 // weights.  A pair's result does not depend on what else is in the step: every output is a dot product
 // over the whole width in a fixed order.
 #include "common.h"
+#include <type_traits>
 
 #define MOE_TILE 64      // pairs of one expert that a workgroup takes (four column tiles of 16)
 #define MOE_KC 128       // inputs per round: the tile's activations of a round meet in LDS
@@ -166,21 +167,28 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restri
     for (int i = 0; i < WLOADS; ++i) *reinterpret_cast<u32x4*>(&wts[piece_row + 16 * i][piece_k]) = wstaged[i];
     __syncthreads();
     if (k0 + MOE_KC < K) fetch(k0 + MOE_KC);  // in flight while this round is multiplied
-    if (n0 < N) {
+    // the round's products in a straight line for the tile's number of column tiles (a test between the
+    // products makes the compiler move the accumulators about: three times the kernel's time)
+    auto multiply = [&](auto count) {
+      constexpr int CT = decltype(count)::value;
 #pragma unroll
       for (int s = 0; s < MOE_KC / 32; ++s) {
         const bf16x8 wv = *reinterpret_cast<const bf16x8*>(&wts[wave * 16 + lr][s * 32 + lg * 8]);
         bf16x8 uv = wv;
         if (GATED) uv = *reinterpret_cast<const bf16x8*>(&wts[MOE_STRIP + wave * 16 + lr][s * 32 + lg * 8]);
 #pragma unroll
-        for (int ct = 0; ct < 4; ++ct) {
-          if (ct < col_tiles) {
-            const bf16x8 av = *reinterpret_cast<const bf16x8*>(&acts[ct * 16 + lr][s * 32 + lg * 8]);
-            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc[ct], 0, 0, 0);
-            if (GATED) acc_up[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv, av, acc_up[ct], 0, 0, 0);
-          }
+        for (int ct = 0; ct < CT; ++ct) {
+          const bf16x8 av = *reinterpret_cast<const bf16x8*>(&acts[ct * 16 + lr][s * 32 + lg * 8]);
+          acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc[ct], 0, 0, 0);
+          if (GATED) acc_up[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv, av, acc_up[ct], 0, 0, 0);
         }
       }
+    };
+    if (n0 < N) {
+      if (col_tiles == 4) multiply(std::integral_constant<int, 4>{});
+      else if (col_tiles == 3) multiply(std::integral_constant<int, 3>{});
+      else if (col_tiles == 2) multiply(std::integral_constant<int, 2>{});
+      else multiply(std::integral_constant<int, 1>{});
     }
   }
   // a lane holds outputs n0 + 4 lg + i (i < 4) of the pair in column lr of each column tile
