@@ -403,9 +403,11 @@ extern "C" int as_delta_finish(const float* o, int H, int vdim, const void* w, i
 // The gates.  u fp32 [T, width] is cut into `blocks` parts of bw channels; in part b
 //   r = sigmoid(ra[b] u_b + ra_b[b]),  i = sigmoid(ri[b] u_b + ri_b[b])     (ra, ri [blocks, bw, bw], out x in)
 //   a = exp(-c r softplus(lam));  a_out = a,  x_out = sqrt(1 - a^2) i u.
-// A workgroup takes 32 tokens by 64 outputs of one part; tokens and weights meet in LDS in pieces of
-// 32 inputs; every output is one fma chain over its inputs in order, whatever shares the launch.
-#define GATE_TT 32
+// A workgroup takes 64 tokens by 64 outputs of one part and a thread four by four of them for both gates;
+// tokens and weights meet in LDS in pieces of 32 inputs, laid out input-major so that a thread reads its
+// four tokens and its four outputs 16 bytes at a time; every output is one fma chain over its inputs in
+// order, whatever shares the launch.
+#define GATE_TT 64
 #define GATE_TO 64
 #define GATE_KC 32
 template <typename W>
@@ -414,50 +416,63 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restric
                                                           const W* __restrict__ ri, const W* __restrict__ ri_b,
                                                           const W* __restrict__ lam, float c, float* __restrict__ a_out,
                                                           float* __restrict__ x_out, int num_tokens) {
-  __shared__ float us[GATE_TT][GATE_KC + 1];
-  __shared__ float wr[GATE_TO][GATE_KC + 1];
-  __shared__ float wi[GATE_TO][GATE_KC + 1];
+  __shared__ __attribute__((aligned(16))) float us[GATE_KC][GATE_TT + 4];
+  __shared__ __attribute__((aligned(16))) float wr[GATE_KC][GATE_TO + 4];
+  __shared__ __attribute__((aligned(16))) float wi[GATE_KC][GATE_TO + 4];
   const int b = blockIdx.y, t0 = blockIdx.x * GATE_TT, o0 = blockIdx.z * GATE_TO;
-  const int tx = threadIdx.x % GATE_TO, ty = threadIdx.x / GATE_TO;  // an output, and 8 of the 32 tokens
-  float accr[8] = {}, acci[8] = {};
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;  // outputs o0 + 4 tx .., tokens t0 + 4 ty ..
+  float accr[4][4] = {}, acci[4][4] = {};
   const W* rab = ra + (size_t)b * bw * bw;
   const W* rib = ri + (size_t)b * bw * bw;
+  const int lk = threadIdx.x & 31, lrow = threadIdx.x >> 5;  // loads: input k0 + lk of rows lrow + 8 i
   for (int k0 = 0; k0 < bw; k0 += GATE_KC) {
-    __syncthreads();
-    for (int e = threadIdx.x; e < GATE_TT * GATE_KC; e += 256) {
-      const int tt = e / GATE_KC, kk = e % GATE_KC;
-      us[tt][kk] = (t0 + tt < num_tokens && k0 + kk < bw) ? u[(size_t)(t0 + tt) * width + b * bw + k0 + kk] : 0.f;
+    float uu[8], rr[8], ii[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = lrow + 8 * i, k = k0 + lk;
+      uu[i] = (t0 + row < num_tokens && k < bw) ? u[(size_t)(t0 + row) * width + b * bw + k] : 0.f;
+      const bool in = o0 + row < bw && k < bw;
+      rr[i] = in ? to_f32(rab[(size_t)(o0 + row) * bw + k]) : 0.f;
+      ii[i] = in ? to_f32(rib[(size_t)(o0 + row) * bw + k]) : 0.f;
     }
-    for (int e = threadIdx.x; e < GATE_TO * GATE_KC; e += 256) {
-      const int oo = e / GATE_KC, kk = e % GATE_KC;
-      const bool in = o0 + oo < bw && k0 + kk < bw;
-      wr[oo][kk] = in ? to_f32(rab[(size_t)(o0 + oo) * bw + k0 + kk]) : 0.f;
-      wi[oo][kk] = in ? to_f32(rib[(size_t)(o0 + oo) * bw + k0 + kk]) : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      us[lk][lrow + 8 * i] = uu[i];
+      wr[lk][lrow + 8 * i] = rr[i];
+      wi[lk][lrow + 8 * i] = ii[i];
     }
     __syncthreads();
 #pragma unroll 8
     for (int kk = 0; kk < GATE_KC; ++kk) {
-      const float a = wr[tx][kk], bb = wi[tx][kk];
+      const float4 u4 = *reinterpret_cast<const float4*>(&us[kk][4 * ty]);
+      const float4 r4 = *reinterpret_cast<const float4*>(&wr[kk][4 * tx]);
+      const float4 i4 = *reinterpret_cast<const float4*>(&wi[kk][4 * tx]);
+      const float uv[4] = {u4.x, u4.y, u4.z, u4.w}, rv[4] = {r4.x, r4.y, r4.z, r4.w}, iv[4] = {i4.x, i4.y, i4.z, i4.w};
 #pragma unroll
-      for (int tt = 0; tt < 8; ++tt) {
-        const float uu = us[ty * 8 + tt][kk];
-        accr[tt] = fmaf(a, uu, accr[tt]);
-        acci[tt] = fmaf(bb, uu, acci[tt]);
-      }
+      for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+        for (int oo = 0; oo < 4; ++oo) {
+          accr[tt][oo] = fmaf(rv[oo], uv[tt], accr[tt][oo]);
+          acci[tt][oo] = fmaf(iv[oo], uv[tt], acci[tt][oo]);
+        }
     }
   }
-  const int o = o0 + tx;
-  if (o >= bw) return;
-  const int ch = b * bw + o;
-  const float rb = to_f32(ra_b[ch]), ib = to_f32(ri_b[ch]), sp = softplusf_(to_f32(lam[ch]));
 #pragma unroll
-  for (int tt = 0; tt < 8; ++tt) {
-    const int t = t0 + ty * 8 + tt;
-    if (t >= num_tokens) continue;
-    const float rg = sigmoidf_(accr[tt] + rb), ig = sigmoidf_(acci[tt] + ib);
-    const float log_a = -c * rg * sp;
-    a_out[(size_t)t * width + ch] = expf(log_a);
-    x_out[(size_t)t * width + ch] = sqrtf(-expm1f(2.0f * log_a)) * ig * u[(size_t)t * width + ch];
+  for (int oo = 0; oo < 4; ++oo) {
+    const int o = o0 + 4 * tx + oo;
+    if (o >= bw) continue;
+    const int ch = b * bw + o;
+    const float rb = to_f32(ra_b[ch]), ib = to_f32(ri_b[ch]), sp = softplusf_(to_f32(lam[ch]));
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+      const int t = t0 + 4 * ty + tt;
+      if (t >= num_tokens) continue;
+      const float rg = sigmoidf_(accr[tt][oo] + rb), ig = sigmoidf_(acci[tt][oo] + ib);
+      const float log_a = -c * rg * sp;
+      a_out[(size_t)t * width + ch] = expf(log_a);
+      x_out[(size_t)t * width + ch] = sqrtf(-expm1f(2.0f * log_a)) * ig * u[(size_t)t * width + ch];
+    }
   }
 }
 
