@@ -136,9 +136,10 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(float* __restrict__ 
                                                             const T* __restrict__ proj, int ld, int b_off, int a_off,
                                                             const W* __restrict__ a_log, const W* __restrict__ dt_bias,
                                                             float* __restrict__ beta, float* __restrict__ decay) {
+  // a workgroup of four waves per token and four heads (blockIdx.y), so that a decode step's few tokens are many workgroups
   const int t = blockIdx.x, lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
   float* row = qkv + (size_t)t * C;
-  for (int head = wave; head < 2 * G; head += waves) {
+  for (int head = blockIdx.y * waves + wave; head < 2 * G; head += gridDim.y * waves) {
     float* x = row + (size_t)head * dim;  // query heads first, then key heads
     float ss = 0.f;
     for (int d = lane; d < dim; d += WAVE) ss += x[d] * x[d];
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(float* __restrict__ 
     if (head < G) f *= 1.0f / sqrtf((float)dim);
     for (int d = lane; d < dim; d += WAVE) x[d] *= f;
   }
-  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+  for (int h = blockIdx.y * blockDim.x + threadIdx.x; h < H; h += gridDim.y * blockDim.x) {
     const float b = to_f32(proj[(size_t)t * ld + b_off + h]), a = to_f32(proj[(size_t)t * ld + a_off + h]);
     beta[(size_t)t * H + h] = sigmoidf_(b);
     decay[(size_t)t * H + h] = expf(-expf(to_f32(a_log[h])) * softplusf_(a + to_f32(dt_bias[h])));
@@ -159,9 +160,11 @@ extern "C" int as_delta_prepare(float* qkv, int C, int G, int dim, int H, const 
                                 float* decay, int num_tokens, hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
   if (G <= 0 || dim <= 0 || H <= 0 || C < 2 * G * dim) return AS_BAD_SHAPE;
+  const int across = num_tokens >= 512 ? 1 : (2 * G + 3) / 4 > 64 ? 64 : (2 * G + 3) / 4;  // many tokens fill the GPU by themselves
+  dim3 grid(num_tokens, across);
 #define LAUNCH(T, W)                                                                                               \
-  delta_prepare_kernel<T, W><<<num_tokens, 256, 0, stream>>>(qkv, C, G, dim, H, (const T*)proj, ld, b_off, a_off,  \
-                                                             (const W*)a_log, (const W*)dt_bias, beta, decay)
+  delta_prepare_kernel<T, W><<<grid, 256, 0, stream>>>(qkv, C, G, dim, H, (const T*)proj, ld, b_off, a_off,        \
+                                                       (const W*)a_log, (const W*)dt_bias, beta, decay)
   if (dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
   else if (dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
   else if (dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
@@ -476,9 +479,10 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restric
   }
 }
 
-// The same for a few tokens (a decode step): the two matrices are streamed once, a wave per output
-// channel, its lanes sharing the inputs (four to a lane per pass, sums over the lanes in a fixed order);
-// four tokens at a time.
+// The same for a few tokens (a decode step): the two matrices are streamed once.  Sixteen lanes share an
+// output channel (a wave four channels): each takes four inputs in sixteen (16-byte loads, a row of the
+// matrix read in whole lines), and their sums meet through DPP moves within the sixteen; eight tokens at a
+// time.  Blocks whose rows do not start on 16 bytes are read value by value.
 template <typename W>
 __global__ __launch_bounds__(256) void rglru_gates_few_kernel(const float* __restrict__ u, int width, int bw,
                                                               const W* __restrict__ ra, const W* __restrict__ ra_b,
@@ -486,28 +490,47 @@ __global__ __launch_bounds__(256) void rglru_gates_few_kernel(const float* __res
                                                               const W* __restrict__ lam, float c,
                                                               float* __restrict__ a_out, float* __restrict__ x_out,
                                                               int num_tokens) {
-  const int lane = threadIdx.x & (WAVE - 1), ch = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-  if (ch >= width) return;
-  const int b = ch / bw, o = ch - b * bw;
+  const int part = threadIdx.x & 15, ch = blockIdx.x * (blockDim.x / 16) + threadIdx.x / 16;
+  const bool mine = ch < width;  // lanes without a channel walk an existing one and store nothing
+  const int chc = mine ? ch : width - 1;
+  const int b = chc / bw, o = chc - b * bw;
   const W* wr = ra + ((size_t)b * bw + o) * bw;
   const W* wi = ri + ((size_t)b * bw + o) * bw;
-  const float rb = to_f32(ra_b[ch]), ib = to_f32(ri_b[ch]), sp = softplusf_(to_f32(lam[ch]));
-  for (int t0 = 0; t0 < num_tokens; t0 += 4) {
-    float accr[4] = {0.f, 0.f, 0.f, 0.f}, acci[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int k = lane; k < bw; k += WAVE) {
-      const float a = to_f32(wr[k]), bb = to_f32(wi[k]);
+  const float rb = to_f32(ra_b[chc]), ib = to_f32(ri_b[chc]), sp = softplusf_(to_f32(lam[chc]));
+  const bool quads = (bw & 3) == 0 && (width & 3) == 0 && sizeof(W) == 4;  // rows start on 16 bytes: four inputs a load
+  for (int t0 = 0; t0 < num_tokens; t0 += 8) {
+    float accr[8] = {}, acci[8] = {};
+    if (quads) {
+      for (int k = 4 * part; k < bw; k += 64) {
+        const float4 a4 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(wr) + k);
+        const float4 b4 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(wi) + k);
+        float4 u4[8];
 #pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
-        const float uu = t0 + tt < num_tokens ? u[(size_t)(t0 + tt) * width + b * bw + k] : 0.f;
-        accr[tt] = fmaf(a, uu, accr[tt]);
-        acci[tt] = fmaf(bb, uu, acci[tt]);
+        for (int tt = 0; tt < 8; ++tt)
+          u4[tt] = t0 + tt < num_tokens ? *reinterpret_cast<const float4*>(u + (size_t)(t0 + tt) * width + b * bw + k)
+                                        : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int tt = 0; tt < 8; ++tt) {
+          accr[tt] = fmaf(a4.w, u4[tt].w, fmaf(a4.z, u4[tt].z, fmaf(a4.y, u4[tt].y, fmaf(a4.x, u4[tt].x, accr[tt]))));
+          acci[tt] = fmaf(b4.w, u4[tt].w, fmaf(b4.z, u4[tt].z, fmaf(b4.y, u4[tt].y, fmaf(b4.x, u4[tt].x, acci[tt]))));
+        }
+      }
+    } else {
+      for (int k = part; k < bw; k += 16) {
+        const float a = to_f32(wr[k]), bb = to_f32(wi[k]);
+#pragma unroll
+        for (int tt = 0; tt < 8; ++tt) {
+          const float uu = t0 + tt < num_tokens ? u[(size_t)(t0 + tt) * width + b * bw + k] : 0.f;
+          accr[tt] = fmaf(a, uu, accr[tt]);
+          acci[tt] = fmaf(bb, uu, acci[tt]);
+        }
       }
     }
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt) {
-      const float sr = wave_sum(accr[tt]), si = wave_sum(acci[tt]);
+    for (int tt = 0; tt < 8; ++tt) {
+      const float sr = slices_sum<16>(accr[tt]), si = slices_sum<16>(acci[tt]);
       const int t = t0 + tt;
-      if (lane == 0 && t < num_tokens) {
+      if (mine && part == 0 && t < num_tokens) {
         const float rg = sigmoidf_(sr + rb), ig = sigmoidf_(si + ib);
         const float log_a = -c * rg * sp;
         a_out[(size_t)t * width + ch] = expf(log_a);
@@ -525,7 +548,7 @@ extern "C" int as_rglru_gates(const float* u, int width, int blocks, const void*
   if (width <= 0 || blocks <= 0 || width % blocks || blocks > 65535) return AS_BAD_SHAPE;
   const int bw = width / blocks;
   if (num_tokens <= GATE_FEW_TOKENS) {
-    const int blocks_few = (width + 3) / 4;
+    const int blocks_few = (width + 15) / 16;  // sixteen channels a workgroup of 256
     if (w_dtype == DT_F32)
       rglru_gates_few_kernel<float><<<blocks_few, 256, 0, stream>>>(u, width, bw, (const float*)ra, (const float*)ra_b,
                                                                    (const float*)ri, (const float*)ri_b,
