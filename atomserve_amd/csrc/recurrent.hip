@@ -331,7 +331,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
 extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int vdim, const float* beta,
                              const float* decay, float* state, const int* row_first, const int* row_len,
                              const int* row_start, const int* row_slots, int writes, float* out, int num_rows,
-                             hipStream_t stream) {
+                             int force_slices, hipStream_t stream) {
   if (num_rows <= 0) return AS_OK;
   if (G <= 0 || H <= 0 || H % G || dim <= 0 || vdim <= 0 || C < 2 * G * dim + H * vdim || H > 65535)
     return AS_BAD_SHAPE;
@@ -342,6 +342,11 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
   while (slices < 16 && (dim + 2 * slices - 1) / (2 * slices) >= 8 &&
          (long)num_rows * H * ((vdim + WAVE / slices - 1) / (WAVE / slices)) < 8L * compute_units())
     slices *= 2;
+  if (force_slices > 0) {  // measurements and tests: 1, 2, 4, 8 or 16 slices, if a lane's share then fits
+    if ((force_slices & (force_slices - 1)) || force_slices > 16 || (dim + force_slices - 1) / force_slices > 64)
+      return AS_BAD_SHAPE;
+    slices = force_slices;
+  }
   const int rows_per_lane = (dim + slices - 1) / slices;
   const int RPL = rows_per_lane <= 8 ? 8 : rows_per_lane <= 16 ? 16 : rows_per_lane <= 32 ? 32 : 64;
   const int CJ = WAVE / slices;

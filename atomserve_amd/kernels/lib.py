@@ -29,7 +29,7 @@ SIGNATURES = {
     "as_sigmoid_gate_heads": ("elementwise", [P, I, I, I, I, P, I, I, F, P, I, I, I, P]),
     "as_short_conv": ("recurrent", [P, I, I, I, I, P, P, P, I, I, I, P, P, P, P, P, P, P, I, I, I, P]),
     "as_delta_prepare": ("recurrent", [P, I, I, I, I, P, I, I, I, I, P, P, I, P, P, I, P]),
-    "as_delta_scan": ("recurrent", [P, I, I, I, I, I, P, P, P, P, P, P, P, I, P, I, P]),
+    "as_delta_scan": ("recurrent", [P, I, I, I, I, I, P, P, P, P, P, P, P, I, P, I, I, P]),
     "as_delta_finish": ("recurrent", [P, I, I, P, I, F, P, I, I, I, P, I, P]),
     "as_rglru_gates": ("recurrent", [P, I, I, P, P, P, P, P, I, F, P, P, I, P]),
     "as_rglru_scan": ("recurrent", [P, P, I, P, I, I, I, P, I, F, P, P, P, P, P, I, P, I, I, I, P]),

@@ -1147,10 +1147,12 @@ def delta_prepare(qkv, num_kv_heads, dim, num_heads, proj, b_off, a_off, a_log, 
          _ptr(dt_bias), _DT[w_dtype], _ptr(beta), _ptr(decay), T, _stream())  # fmt: skip
 
 
-def delta_scan(qkv, num_kv_heads, dim, num_heads, vdim, beta, decay, state, step_rows, out, writes=True) -> None:
+def delta_scan(qkv, num_kv_heads, dim, num_heads, vdim, beta, decay, state, step_rows, out, writes=True, slices=0) -> None:
     """The gated delta rule over each row's tokens, per head h (keys and queries of head h // (H / G)):
     S <- decay S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.  state fp32 [slots, H, dim, vdim]; a row
-    that starts at position 0 starts from zero.  qkv as `delta_prepare` left it; out fp32 [T, H, vdim]."""
+    that starts at position 0 starts from zero.  qkv as `delta_prepare` left it; out fp32 [T, H, vdim].
+    slices: into how many lanes a column of the state is cut (1, 2, 4, 8, 16); 0: chosen so that the step's rows,
+    heads and column groups fill the GPU (the results differ by the order of the sums only)."""
     _check(qkv, "qkv", F32, (None, None))
     T, C = qkv.shape
     G, H = num_kv_heads, num_heads
@@ -1163,7 +1165,7 @@ def delta_scan(qkv, num_kv_heads, dim, num_heads, vdim, beta, decay, state, step
     R = _check_rows((None, *step_rows[1:]), 0)
     _, row_first, row_len, row_start, row_slots = step_rows
     call("as_delta_scan", _ptr(qkv), C, G, dim, H, vdim, _ptr(beta), _ptr(decay), _ptr(state), _ptr(row_first),
-         _ptr(row_len), _ptr(row_start), _ptr(row_slots), int(bool(writes)), _ptr(out), R, _stream())  # fmt: skip
+         _ptr(row_len), _ptr(row_start), _ptr(row_slots), int(bool(writes)), _ptr(out), R, int(slices), _stream())  # fmt: skip
 
 
 def delta_finish(o, weight, eps, proj, g_off, act) -> None:

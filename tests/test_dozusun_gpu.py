@@ -258,6 +258,46 @@ def test_delta_rule_alone(shape, dtype):
         assert (got - ref).abs().max() <= tol, f"{shape} {cuts}: {float((got - ref).abs().max()):.3e} of {float(ref.abs().max()):.3e}"
 
 
+@pytest.mark.parametrize("dim,vdim", [(128, 128), (64, 40), (24, 72), (200, 16)])
+def test_delta_scan_however_the_state_is_cut_over_lanes(dim, vdim):
+    """The scan cuts a column of the state into 1 to 16 slices by how many rows and heads a step has; every cut that
+    a width allows gives the recurrence's result, from a state that another request left and over several rows."""
+    from atomserve_amd.kernels import ops
+
+    H, G, gen = 3, 1, torch.Generator().manual_seed(dim + vdim)
+    lens, starts, slots = [9, 1, 17], [0, 5, 0], [2, 0, 1]
+    T, C = sum(lens), 2 * G * dim + H * vdim
+    qkv = torch.randn(T, C, generator=gen)
+    qkv[:, : 2 * G * dim] *= dim**-0.5
+    beta, decay = torch.rand(T, H, generator=gen), 0.5 + 0.5 * torch.rand(T, H, generator=gen)
+    state0 = torch.randn(4, H, dim, vdim, generator=gen)
+    want, at = torch.zeros(T, H, vdim, dtype=torch.float64), 0
+    final = state0.double().clone()
+    for n, start, slot in zip(lens, starts, slots):
+        for h in range(H):
+            S = final[slot, h].clone() if start > 0 else torch.zeros(dim, vdim, dtype=torch.float64)
+            for t in range(at, at + n):
+                q, k, v = qkv[t, :dim].double(), qkv[t, dim : 2 * dim].double(), qkv[t, 2 * dim + h * vdim : 2 * dim + (h + 1) * vdim].double()
+                S = decay[t, h].double() * S
+                S = S + torch.outer(k, beta[t, h].double() * (v - S.T @ k))
+                want[t, h] = S.T @ q
+            final[slot, h] = S
+        at += n
+    firsts = [sum(lens[:i]) for i in range(len(lens))]
+    rows = (None,) + tuple(torch.tensor(v, dtype=torch.int32, device=DEV) for v in (firsts, lens, starts, slots))
+    tried = 0
+    for slices in (0, 1, 2, 4, 8, 16):
+        if slices and -(-dim // slices) > 64:
+            continue
+        state = state0.clone().to(DEV)
+        out = torch.empty((T, H, vdim), dtype=torch.float32, device=DEV)
+        ops.delta_scan(qkv.to(DEV), G, dim, H, vdim, beta.to(DEV), decay.to(DEV), state, rows, out, slices=slices)
+        assert (out.cpu().double() - want).abs().max() <= 2e-5 * float(want.abs().max()), f"{slices} slices"
+        assert (state.cpu().double() - final).abs().max() <= 2e-5 * float(final.abs().max()), f"{slices} slices: the state"
+        tried += 1
+    assert tried >= 4
+
+
 def test_delta_rule_keeps_a_far_token():
     """With a decay near one and a query that asks for one early token's key, the output hundreds of tokens later
     is that token's value: a state that was lost or restarted on the way shows as a difference of the output's size."""
@@ -408,8 +448,9 @@ def test_attention_without_a_window_finds_a_far_key_among_hundreds(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("experts,top,ff,T", [(5, 2, 24, 70), (3, 3, 8, 5), (9, 1, 40, 33), (2, 1, 16, 1)])
+@pytest.mark.parametrize("experts,top,ff,T", [(5, 2, 24, 70), (3, 3, 8, 5), (9, 1, 40, 33), (2, 1, 16, 1), (2, 1, 16, 200), (3, 2, 8, 150)])
 def test_table_routed_experts_alone(experts, top, ff, T, dtype):
+    """From one pair to an expert up to a hundred (several tiles of 64 pairs, the last one partly filled)."""
     from atomserve_amd.engine.batch import Row, StepBatch
     from atomserve_amd.parts.base import build
     from atomserve_amd.parts.plan import TableExpertsSpec
