@@ -152,10 +152,11 @@ class CacheManager:
                 continue
             first_visible = num_computed - g.window + 1  # the oldest key the next query sees
             dead = min(len(table), max(0, first_visible) // self.block_size)
-            pages = [table[b] for b in range(dead) if table[b] != RELEASED]
+            kept = blocks_for_tokens(g.request.keep_first, self.block_size)  # pages of tokens that stay visible for good
+            pages = [table[b] for b in range(kept, dead) if table[b] != RELEASED]
             if pages:
                 g.allocator.free(pages)
-                for b in range(dead):
+                for b in range(kept, dead):
                     table[b] = RELEASED
                 freed += len(pages)
         return freed

@@ -286,3 +286,172 @@ class DozusunConfig:
         if self.loop_times > 1 or self.loop_stop > self.loop_start:
             raw["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
         return raw
+
+
+# ---- Koravik ------------------------------------------------------------------------------------------
+
+
+@dataclass(frozen=True)
+class KoravikAttention:
+    """An attention mixer's sizes and constants."""
+
+    heads: int
+    kv_heads: int
+    dim: int  # width of a query/key head
+    vdim: int  # width of a value head: the keys are the values, so this is `dim`
+    scale: float  # multiplies q.k
+    rot_dims: int  # coordinates of a head that turn with the position
+    rot_base: float
+    window: int  # keys a position sees, itself included
+    keep_first: int  # the sequence's first tokens, which stay visible behind the window
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "KoravikAttention":
+        rot, mask = _need(raw, "rot", where), _need(raw, "mask", where)
+        return cls(
+            heads=int(_need(raw, "heads", where)),
+            kv_heads=int(_need(raw, "kv_heads", where)),
+            dim=int(_need(raw, "dim", where)),
+            vdim=int(raw.get("vdim", raw.get("dim", 0))),
+            scale=float(_need(raw, "scale", where)),
+            rot_dims=int(_need(rot, "dims", where + "rot.")),
+            rot_base=float(_need(rot, "base", where + "rot.")),
+            window=int(_need(mask, "size", where + "mask.")),
+            keep_first=int(mask.get("keep_first", 0)),
+        )
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale,
+                "rot": {"dims": self.rot_dims, "base": self.rot_base},
+                "mask": {"size": self.window, "keep_first": self.keep_first}}  # fmt: skip
+
+
+@dataclass(frozen=True)
+class KoravikExperts:
+    """A feed-forward of routed experts with one shared expert (shared_ff 0: none)."""
+
+    ff: int  # width inside one expert
+    experts: int
+    top: int
+    shared_ff: int
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "KoravikExperts":
+        kind = _need(raw, "kind", where)
+        if kind != "moe":
+            raise ConfigError(f"{where}kind={kind!r} is not supported (only 'moe')")
+        router = _need(raw, "router", where)
+        shared = raw.get("shared") or {}
+        return cls(
+            ff=int(_need(_need(raw, "expert", where), "ff", where + "expert.")),
+            experts=int(_need(router, "experts", where + "router.")),
+            top=int(_need(router, "top", where + "router.")),
+            shared_ff=int(shared.get("ff", 0)),
+        )
+
+    def to_dict(self) -> dict:
+        raw = {"kind": "moe", "expert": {"ff": self.ff}, "router": {"experts": self.experts, "top": self.top}}
+        if self.shared_ff:
+            raw["shared"] = {"ff": self.shared_ff}
+        return raw
+
+
+@dataclass(frozen=True)
+class KoravikLayer:
+    type: str  # "attention"
+    mixer: KoravikAttention
+    mlp: object  # KoravikExperts or None
+
+
+@dataclass(frozen=True)
+class KoravikConfig:
+    """A Koravik decoder: pre-norm layers of a mixed-heads attention and routed experts whose outputs enter the
+    stream through a sigmoid gate and a common factor; the embedding is normed; a stretch of layers may run
+    several times in a row, each pass entering through a matrix that also reads the embedding's output; the
+    head is the embedding table, its logits scaled."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    residual_mult: float
+    logit_scale: float
+    layers: tuple  # of KoravikLayer
+    loop: bool = False  # whether a stretch is looped (and `loop.in` exists)
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+
+    architecture = "Koravik"
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "KoravikConfig":
+        _require(raw, ["vocab", "width", "layers", "norm", "residual_mult", "logit_scale"])
+        layers = []
+        for i, entry in enumerate(raw["layers"]):
+            where = f"layers[{i}]."
+            kind = _need(entry, "type", where)
+            if kind != "attention":
+                raise ConfigError(f"{where}type={kind!r} is not supported (only 'attention')")
+            mixer = KoravikAttention.from_dict(_need(entry, "mixer", where), where + "mixer.")
+            mlp = entry.get("mlp")
+            layers.append(KoravikLayer(kind, mixer, None if mlp is None else KoravikExperts.from_dict(mlp, where + "mlp.")))
+        loop = raw.get("loop")
+        cfg = cls(
+            vocab_size=int(raw["vocab"]),
+            hidden_size=int(raw["width"]),
+            norm_eps=float(_need(raw["norm"], "eps", "norm.")),
+            residual_mult=float(raw["residual_mult"]),
+            logit_scale=float(raw["logit_scale"]),
+            layers=tuple(layers),
+            loop=bool(loop),
+            loop_start=int(_need(loop, "start", "loop.")) if loop else 0,
+            loop_stop=int(_need(loop, "stop", "loop.")) if loop else 0,
+            loop_times=int(_need(loop, "times", "loop.")) if loop else 1,
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size < 1 or self.hidden_size < 1 or not self.layers:
+            raise ConfigError("vocab, width and the number of layers must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        if not 0 <= self.loop_start <= self.loop_stop <= len(self.layers) or self.loop_times < 1:
+            raise ConfigError(f"loop {self.loop_start}:{self.loop_stop} x {self.loop_times} does not fit {len(self.layers)} layers")
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            if min(m.heads, m.kv_heads, m.dim) < 1 or m.heads % m.kv_heads:
+                raise ConfigError(f"layers[{i}]: head counts and sizes must be positive, heads a multiple of kv_heads")
+            if m.vdim != m.dim:
+                raise ConfigError(f"layers[{i}]: the values are the keys, so vdim {m.vdim} must equal dim {m.dim}")
+            if m.rot_dims < 0 or m.rot_dims % 2 or m.rot_dims > m.dim or not m.rot_base > 0:
+                raise ConfigError(f"layers[{i}]: rot.dims must be even and at most dim, rot.base positive")
+            if m.window < 1 or m.keep_first < 0:
+                raise ConfigError(f"layers[{i}]: mask.size must be positive and mask.keep_first not negative")
+            f = layer.mlp
+            if f is not None and (f.ff < 1 or f.shared_ff < 0 or not 1 <= f.top <= f.experts):
+                raise ConfigError(f"layers[{i}].mlp: sizes must be positive and top at most the number of experts")
+
+    def run_order(self) -> list:
+        """(layer, whether the stream re-enters before it) in the order the layers run: the looped stretch
+        `times` times, every pass entering through the loop's matrix before its first layer."""
+        n = len(self.layers)
+        order = [(i, False) for i in range(self.loop_start)]
+        for _ in range(self.loop_times if self.loop else 0):
+            order += [(i, i == self.loop_start) for i in range(self.loop_start, self.loop_stop)]
+        return order + [(i, False) for i in range(self.loop_stop if self.loop else 0, n)]
+
+    @property
+    def reenters(self) -> bool:
+        return any(r for _, r in self.run_order())
+
+    def to_dict(self) -> dict:
+        """The config.json that `from_dict` reads back to this object."""
+        layers = [{"type": layer.type, "mixer": layer.mixer.to_dict(), "mlp": None if layer.mlp is None else layer.mlp.to_dict()}
+                  for layer in self.layers]  # fmt: skip
+        raw = {"architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+               "norm": {"eps": self.norm_eps}, "residual_mult": self.residual_mult, "logit_scale": self.logit_scale,
+               "layers": layers}  # fmt: skip
+        if self.loop:
+            raw["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
+        return raw

@@ -22,8 +22,8 @@ class Architecture:
     checkpoint_map: typed configuration -> {plan tensor name: [checkpoint names to stack]}
     checkpoint_shapes: typed configuration -> {checkpoint name: (shape, role)}, in the order in which
                     random weights are drawn; roles: "matrix", "vector" (gains around 1), "bias" and
-                    "log_rate" (small values around 0), "expert_table:<experts>" (int32 rows of distinct
-                    expert numbers)
+                    "log_rate" (small values around 0), "near_identity" (a square matrix around the
+                    identity), "expert_table:<experts>" (int32 rows of distinct expert numbers)
     ignored:        typed configuration -> checkpoint names that may be present and unused
     """
 
@@ -78,4 +78,5 @@ def load_model_config(model_dir: str) -> tuple[Architecture, Any]:
 def _load_builtin() -> None:
     # Imported lazily: the model modules import parts, which import this package.
     import atomserve_amd.models.dozusun  # noqa: F401
+    import atomserve_amd.models.koravik  # noqa: F401
     import atomserve_amd.models.qwen3  # noqa: F401

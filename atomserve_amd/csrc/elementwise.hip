@@ -589,7 +589,9 @@ extern "C" int as_rmsnorm_multi(float* x, const void* d1, const void* d2, const 
 // ---- heads out of a wider projection: per-head norm, padding, cache store ------------------
 // proj [T, ld] holds, among other columns, H query heads and KV key heads of `dim` coordinates and KV
 // value heads of `vdim`, starting at columns q_off, k_off, v_off.  Queries and keys are normed per head
-// (x / sqrt(mean(x^2) + eps) * weight over dim; no weights: left as they are); nothing is rotated.
+// (x / sqrt(mean(x^2) + eps) * weight over dim; no weights: left as they are), then turned if a table of
+// angles comes with them (cs [T, R/2] of (cos, sin): the pairs (i, i + R/2) of a head's first R coordinates, as
+// in qk_norm_rope_store; values are never turned, so values read from the keys' columns are the keys unturned).
 // The attention kernels take one head width for keys and values, so every head is laid out with
 // Dp >= max(dim, vdim) coordinates, the ones a head does not have being zero: scores and outputs are
 // unchanged.  q_out [T, H, Dp]; keys to k_pages [pages, KV, bs, Dp] and values transposed to v_pages
@@ -600,7 +602,8 @@ __global__ __launch_bounds__(64) void head_norm_store_kernel(const T* __restrict
                                                              const W* __restrict__ qw, const W* __restrict__ kw,
                                                              float eps, const int* __restrict__ slots,
                                                              T* __restrict__ q_out, T* __restrict__ k_pages,
-                                                             T* __restrict__ v_pages, int bs, int store) {
+                                                             T* __restrict__ v_pages, int bs, int store,
+                                                             const float2* __restrict__ cs, int R) {
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const T* row = proj + (size_t)t * ld;
   if (head < H + KV) {  // a query or a key head
@@ -623,9 +626,16 @@ __global__ __launch_bounds__(64) void head_norm_store_kernel(const T* __restrict
       ss = wave_sum(ss);
       inv = 1.0f / sqrtf(ss / (float)dim + eps);
     }
+    const int half = cs ? R / 2 : 0;
     for (int d = lane; d < Dp; d += WAVE) {
       float v = 0.f;
       if (d < dim) v = w ? to_f32(src[d]) * inv * to_f32(w[d]) : to_f32(src[d]);
+      if (d < 2 * half) {  // the partner of coordinate d, and the turn by the token's angle
+        const int i = d < half ? d : d - half, o = d < half ? d + half : d - half;
+        const float u = w ? to_f32(src[o]) * inv * to_f32(w[o]) : to_f32(src[o]);
+        const float2 a = cs[(size_t)t * half + i];
+        v = d < half ? v * a.x - u * a.y : v * a.x + u * a.y;
+      }
       dst[d] = from_f32<T>(finite_or_zero(v));
     }
     return;
@@ -641,8 +651,9 @@ __global__ __launch_bounds__(64) void head_norm_store_kernel(const T* __restrict
 extern "C" int as_head_norm_store(const void* proj, int dtype, int ld, int q_off, int k_off, int v_off, int H, int KV,
                                   int dim, int vdim, int Dp, const void* qw, const void* kw, int w_dtype, float eps,
                                   const int* slots, void* q_out, void* k_pages, void* v_pages, int bs, int store,
-                                  int num_tokens, hipStream_t stream) {
+                                  int num_tokens, const float* cs, int R, hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
+  if (cs && (R <= 0 || (R & 1) || R > dim)) return AS_BAD_SHAPE;
   if (H <= 0 || KV <= 0 || dim <= 0 || vdim <= 0 || Dp < dim || Dp < vdim || bs <= 0 || ld <= 0 || (!qw) != (!kw))
     return AS_BAD_SHAPE;
   if (H + 2 * KV > 65535) return AS_BAD_SHAPE;
@@ -650,7 +661,8 @@ extern "C" int as_head_norm_store(const void* proj, int dtype, int ld, int q_off
 #define LAUNCH(T, W)                                                                                          \
   head_norm_store_kernel<T, W><<<grid, 64, 0, stream>>>((const T*)proj, ld, q_off, k_off, v_off, H, KV, dim,  \
                                                         vdim, Dp, (const W*)qw, (const W*)kw, eps, slots,     \
-                                                        (T*)q_out, (T*)k_pages, (T*)v_pages, bs, store)
+                                                        (T*)q_out, (T*)k_pages, (T*)v_pages, bs, store,       \
+                                                        (const float2*)cs, R)
   if (dtype == DT_F32 && (w_dtype == DT_F32 || !qw)) LAUNCH(float, float);
   else if (dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
   else if (dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
@@ -691,6 +703,100 @@ extern "C" int as_sigmoid_gate_heads(const void* heads, int dtype, int H, int vd
   else if (dtype == DT_BF16)
     sigmoid_gate_heads_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)heads, H, vdim, Dp, (const bf16*)gate,
                                                                 ld_gate, gate_off, scale, (bf16*)out, ld_out, out_off, total);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// ---- a gated, scaled residual sum, with the norm that follows it -------------------------------
+// For source row s (= rows ? rows[r] : r) of the fp32 stream x [T, n]:
+//   v = x[s] + mult * sigmoid(gate[s, gate_off + i] + bias[i]) * y[s, i]      (y null: v = x[s]); written back if update_x
+//   out[r]  = v / sqrt(mean(v^2) + eps) * w, rounded once                     (w null: no norm is taken)
+//   join[r] = [ v | other[s] ] rounded to O, 2n wide                           (join null: none)
+// y and gate are a part's output and the logits of its output gate (columns of a wider product, ld_gate wide);
+// the sum and the sigmoid are fp32.  `join` hands the stream, beside another fp32 stream, to a product that
+// takes both.
+template <typename O, typename W, typename NO>
+__global__ void gated_add_norm_kernel(float* __restrict__ x, const O* __restrict__ y, const O* __restrict__ gate,
+                                      int ld_gate, int gate_off, const W* __restrict__ bias, float mult,
+                                      const int* __restrict__ rows, const W* __restrict__ w, float eps,
+                                      NO* __restrict__ out, int n, int update_x, const float* __restrict__ other,
+                                      O* __restrict__ join) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const size_t s = rows ? (size_t)rows[r] : (size_t)r;
+  float* xr = x + s * n;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = xr[i];
+    if (y) {
+      const float g = to_f32(gate[s * ld_gate + gate_off + i]) + (bias ? to_f32(bias[i]) : 0.f);
+      v += mult * to_f32(y[s * n + i]) / (1.0f + expf(-g));
+      if (update_x) xr[i] = v;
+    }
+    ss += v * v;
+    if (join) {
+      join[(size_t)r * 2 * n + i] = from_f32<O>(v);
+      join[(size_t)r * 2 * n + n + i] = from_f32<O>(other[s * n + i]);
+    }
+  }
+  if (!w) return;
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+  NO* o = out + (size_t)r * n;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = xr[i];  // the thread's own earlier store, if any, is what it reads back
+    if (y && !update_x) {
+      const float g = to_f32(gate[s * ld_gate + gate_off + i]) + (bias ? to_f32(bias[i]) : 0.f);
+      v += mult * to_f32(y[s * n + i]) / (1.0f + expf(-g));
+    }
+    o[i] = from_f32<NO>(v * inv * to_f32(w[i]));
+  }
+}
+
+// dtype: of y, gate and join; w_dtype: of bias and w; out_dtype: of out (fp32 for a norm whose result is a stream).
+extern "C" int as_gated_add_norm(float* x, const void* y, const void* gate, int dtype, int ld_gate, int gate_off,
+                                 const void* bias, float mult, const int* rows, const void* w, int w_dtype, float eps,
+                                 void* out, int out_dtype, int n_out, int n, int update_x, const float* other,
+                                 void* join, hipStream_t stream) {
+  if (n_out <= 0) return AS_OK;
+  if (n <= 0 || (y && (!gate || ld_gate < n || gate_off < 0 || gate_off + n > ld_gate)) || (w && !out) ||
+      (join && !other))
+    return AS_BAD_SHAPE;
+  const int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : 64);
+#define LAUNCH(O, W, NO)                                                                                          \
+  gated_add_norm_kernel<O, W, NO><<<n_out, threads, 0, stream>>>(x, (const O*)y, (const O*)gate, ld_gate, gate_off, \
+                                                                 (const W*)bias, mult, rows, (const W*)w, eps,      \
+                                                                 (NO*)out, n, update_x, other, (O*)join)
+  if (dtype == DT_F32 && w_dtype == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float, float);
+  else if (dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_BF16) LAUNCH(bf16, bf16, bf16);
+  else if (dtype == DT_BF16 && w_dtype == DT_F32 && out_dtype == DT_BF16) LAUNCH(bf16, float, bf16);
+  else if (dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_F32) LAUNCH(bf16, bf16, float);
+  else if (dtype == DT_BF16 && w_dtype == DT_F32 && out_dtype == DT_F32) LAUNCH(bf16, float, float);
+  else return AS_BAD_DTYPE;
+#undef LAUNCH
+  return launch_status();
+}
+
+// ---- relu(x)^2 on the first columns of a wider product --------------------------------------------
+// out[t, i] = max(a[t, off + i], 0)^2 for i < n; a [T, ld].
+template <typename T>
+__global__ void relu2_kernel(const T* __restrict__ a, int ld, int off, T* __restrict__ out, int n, size_t total) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    const size_t t = idx / n;
+    const float v = fmaxf(to_f32(a[t * ld + off + idx % n]), 0.f);
+    out[idx] = from_f32<T>(v * v);
+  }
+}
+
+extern "C" int as_relu2(const void* a, int dtype, int ld, int off, void* out, int n, int num_tokens,
+                        hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (n <= 0 || off < 0 || off + n > ld) return AS_BAD_SHAPE;
+  const size_t total = (size_t)num_tokens * n, want = (total + 255) / 256;
+  const int blocks = (int)(want > 8192 ? 8192 : want);
+  if (dtype == DT_F32) relu2_kernel<float><<<blocks, 256, 0, stream>>>((const float*)a, ld, off, (float*)out, n, total);
+  else if (dtype == DT_BF16) relu2_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)a, ld, off, (bf16*)out, n, total);
   else return AS_BAD_DTYPE;
   return launch_status();
 }

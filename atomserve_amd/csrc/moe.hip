@@ -25,6 +25,20 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes as 
 // tiles [max_tiles, 3]: (expert, first place in `order`, count <= 64); counts[0] = number of tiles.
 // One workgroup; the order of pairs within an expert is whatever the atomics make it, which no
 // result depends on.
+// With token_ids null, `table` is [P]: the expert of every pair as a router's kernel left it.
+__device__ __forceinline__ int expert_of_pair(const int* token_ids, const int* table, int vocab, int top, int experts,
+                                              int p) {
+  int e;
+  if (token_ids) {
+    int id = token_ids[p / top];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    e = table[(size_t)id * top + p % top];
+  } else {
+    e = table[p];
+  }
+  return e < 0 ? 0 : (e >= experts ? experts - 1 : e);
+}
+
 __global__ __launch_bounds__(1024) void moe_route_table_kernel(const int* __restrict__ token_ids,
                                                                const int* __restrict__ table, int vocab, int top,
                                                                int experts, int num_tokens, int* __restrict__ order,
@@ -36,10 +50,7 @@ __global__ __launch_bounds__(1024) void moe_route_table_kernel(const int* __rest
   for (int e = threadIdx.x; e < experts; e += blockDim.x) hist[e] = 0;
   __syncthreads();
   for (int p = threadIdx.x; p < P; p += blockDim.x) {
-    int id = token_ids[p / top];
-    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
-    int e = table[(size_t)id * top + p % top];
-    e = e < 0 ? 0 : (e >= experts ? experts - 1 : e);
+    const int e = expert_of_pair(token_ids, table, vocab, top, experts, p);
     atomicAdd(&hist[e], 1);
   }
   __syncthreads();
@@ -58,19 +69,90 @@ __global__ __launch_bounds__(1024) void moe_route_table_kernel(const int* __rest
   }
   __syncthreads();
   for (int p = threadIdx.x; p < P; p += blockDim.x) {
-    int id = token_ids[p / top];
-    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
-    int e = table[(size_t)id * top + p % top];
-    e = e < 0 ? 0 : (e >= experts ? experts - 1 : e);
+    const int e = expert_of_pair(token_ids, table, vocab, top, experts, p);
     order[atomicAdd(&cursor[e], 1)] = p;
   }
+}
+
+// ---- a router that scores every expert ---------------------------------------------------------------
+// z = router h in fp32 (router [experts, K], h [T, K], both T-typed), s = sigmoid(z); a token's `top` experts are
+// those with the largest s (of equal ones the lower number first); their weights are s / (sum of the chosen + 1e-20).
+// pair_expert, pair_weight [T * top].  A wave per token: every lane walks the width in strides for one expert
+// after the other, the sums meet by lane swaps, the choice runs over LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(const T* __restrict__ h, const T* __restrict__ router,
+                                                                int K, int experts, int top, int num_tokens,
+                                                                int* __restrict__ pair_expert,
+                                                                float* __restrict__ pair_weight) {
+  extern __shared__ float scores[];  // [4][experts]
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= num_tokens) return;
+  float* mine = scores + (size_t)wave * experts;
+  const T* row = h + (size_t)t * K;
+  for (int e = 0; e < experts; ++e) {
+    const T* wr = router + (size_t)e * K;
+    float z = 0.f;
+    for (int k = lane; k < K; k += WAVE) z = fmaf(to_f32(row[k]), to_f32(wr[k]), z);
+    z = wave_sum(z);
+    if (lane == 0) mine[e] = 1.0f / (1.0f + expf(-z));
+  }
+  __builtin_amdgcn_wave_barrier();
+  float total = 0.f, my_score = 0.f;
+  int my_expert = 0;
+  for (int j = 0; j < top; ++j) {
+    float best = -1.f;
+    int at = 0x7fffffff;
+    for (int e = lane; e < experts; e += WAVE) {
+      const float v = mine[e];
+      if (v > best) { best = v; at = e; }
+    }
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, WAVE);
+      const int oa = __shfl_xor(at, off, WAVE);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    if (at >= experts) { at = 0; best = 0.f; }  // nothing left to choose (scores that are not numbers)
+    if (lane == j % WAVE && j / WAVE == 0) { my_score = best; my_expert = at; }
+    if (j >= WAVE && lane == 0) {  // more than 64 experts a token: written as they are found, weighed below
+      pair_expert[(size_t)t * top + j] = at;
+      pair_weight[(size_t)t * top + j] = best;
+    }
+    total += best;
+    if (lane == 0) mine[at] = -2.f;
+    __builtin_amdgcn_wave_barrier();
+  }
+  const float inv = 1.0f / (total + 1e-20f);
+  if (lane < top && lane < WAVE) {
+    pair_expert[(size_t)t * top + lane] = my_expert;
+    pair_weight[(size_t)t * top + lane] = my_score * inv;
+  }
+  if (lane == 0)
+    for (int j = WAVE; j < top; ++j) pair_weight[(size_t)t * top + j] *= inv;
+}
+
+extern "C" int as_moe_route_sigmoid(const void* h, const void* router, int dtype, int K, int experts, int top,
+                                    int num_tokens, int* pair_expert, float* pair_weight, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (K <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts) return AS_BAD_SHAPE;
+  const int blocks = (num_tokens + 3) / 4;
+  const size_t lds = (size_t)4 * experts * sizeof(float);
+  if (dtype == DT_F32)
+    moe_route_sigmoid_kernel<float><<<blocks, 256, lds, stream>>>((const float*)h, (const float*)router, K, experts, top,
+                                                                  num_tokens, pair_expert, pair_weight);
+  else if (dtype == DT_BF16)
+    moe_route_sigmoid_kernel<bf16><<<blocks, 256, lds, stream>>>((const bf16*)h, (const bf16*)router, K, experts, top,
+                                                                 num_tokens, pair_expert, pair_weight);
+  else return AS_BAD_DTYPE;
+  return launch_status();
 }
 
 extern "C" int as_moe_route_table(const int* token_ids, const int* table, int vocab, int top, int experts,
                                   int num_tokens, int* order, int* tiles, int* counts, int max_tiles,
                                   hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
-  if (top <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || vocab <= 0) return AS_BAD_SHAPE;
+  if (top <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || (token_ids && vocab <= 0)) return AS_BAD_SHAPE;
   if (max_tiles < (num_tokens * top + MOE_TILE - 1) / MOE_TILE + experts) return AS_BAD_SHAPE;
   moe_route_table_kernel<<<1, 1024, 0, stream>>>(token_ids, table, vocab, top, experts, num_tokens, order, tiles,
                                                  counts, max_tiles);
@@ -98,7 +180,7 @@ __device__ __forceinline__ bf16x8 row_piece(const bf16* row, int k, int K) {
   return v;
 }
 
-template <bool GATED, typename OutT>
+template <bool GATED, typename OutT, bool RELU2 = false>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restrict__ a, int a_div,
                                                             const bf16* __restrict__ w, int N, int K,
                                                             const int* __restrict__ order,
@@ -207,6 +289,10 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restri
         const float g = to_f32((bf16)acc[ct][i]), u = to_f32((bf16)acc_up[ct][i]);  // the two products rounded as if stored
         v = g / (1.0f + expf(-g)) * u;
       }
+      if (RELU2) {
+        const float u = fmaxf(to_f32((bf16)v), 0.f);  // the product rounded as if stored
+        v = u * u;
+      }
       out[(size_t)pair * N + n] = from_f32<OutT>(v);
     }
   }
@@ -214,7 +300,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restri
 
 // fp32: plain multiply-add, every output one chain over k in order.  A thread owns an output and, of every
 // sixteen of the tile's pairs in turn, four.
-template <bool GATED>
+template <bool GATED, bool RELU2 = false>
 __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(const float* __restrict__ a, int a_div,
                                                            const float* __restrict__ w, int N, int K,
                                                            const int* __restrict__ order,
@@ -253,6 +339,7 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(const float* __restri
       if (pairs[i] < 0) continue;
       float v = acc[i];
       if (GATED) v = v / (1.0f + expf(-v)) * acc_up[i];
+      if (RELU2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
       out[(size_t)pairs[i] * N + n] = v;
     }
   }
@@ -260,6 +347,7 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(const float* __restri
 
 // out_dtype: DT_BF16 or DT_F32 for the bf16 product's results (fp32 where several experts' outputs
 // are still to be added up); the fp32 product writes fp32.
+// gated: 0: the product; 1: silu(gate) * up; 2: relu(product)^2 (an expert without a gate).
 extern "C" int as_moe_gemm(const void* a, int dtype, int a_div, const void* w, int N, int K, int gated, const int* order,
                            const int* tiles, const int* counts, int max_tiles, void* out, int out_dtype,
                            hipStream_t stream) {
@@ -268,12 +356,16 @@ extern "C" int as_moe_gemm(const void* a, int dtype, int a_div, const void* w, i
   dim3 grid((N + MOE_STRIP - 1) / MOE_STRIP, max_tiles);
   if (dtype == DT_F32) {
     if (out_dtype != DT_F32) return AS_BAD_DTYPE;
-    if (gated) moe_gemm_f32_kernel<true><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out);
+    if (gated == 2) moe_gemm_f32_kernel<false, true><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out);
+    else if (gated) moe_gemm_f32_kernel<true><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out);
     else moe_gemm_f32_kernel<false><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out);
     return launch_status();
   }
   if (dtype != DT_BF16) return AS_BAD_DTYPE;
-  if (gated) {
+  if (gated == 2) {
+    if (out_dtype != DT_BF16) return AS_BAD_DTYPE;
+    moe_gemm_bf16_kernel<false, bf16, true><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out);
+  } else if (gated) {
     if (out_dtype != DT_BF16) return AS_BAD_DTYPE;
     moe_gemm_bf16_kernel<true, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out);
   } else if (out_dtype == DT_BF16) {
@@ -286,28 +378,32 @@ extern "C" int as_moe_gemm(const void* a, int dtype, int a_div, const void* w, i
   return launch_status();
 }
 
-// out[t, n] = sum over a token's `top` pairs of weight * pair_out[t * top + j, n]  (fp32 in, T out).
+// out[t, n] = sum over a token's `top` pairs of weight * pair_weight[t * top + j] * pair_out[t * top + j, n]
+// (+ add[t, n]); fp32 in, T out.  pair_weight null: every pair weighs `weight`; add (T) null: nothing is added.
 template <typename T>
 __global__ void moe_combine_kernel(const float* __restrict__ pair_out, int top, float weight, int N,
-                                   T* __restrict__ out, size_t total) {
+                                   T* __restrict__ out, size_t total, const float* __restrict__ pair_weight,
+                                   const T* __restrict__ add) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
     const size_t t = idx / N;
     const int n = (int)(idx % N);
     float s = 0.f;
-    for (int j = 0; j < top; ++j) s += weight * pair_out[(t * top + j) * N + n];
+    for (int j = 0; j < top; ++j)
+      s += weight * (pair_weight ? pair_weight[t * top + j] : 1.f) * pair_out[(t * top + j) * N + n];
+    if (add) s += to_f32(add[idx]);
     out[idx] = from_f32<T>(s);
   }
 }
 
 extern "C" int as_moe_combine(const float* pair_out, int top, float weight, int N, void* out, int out_dtype,
-                              int num_tokens, hipStream_t stream) {
+                              int num_tokens, const float* pair_weight, const void* add, hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
   if (top <= 0 || N <= 0) return AS_BAD_SHAPE;
   const size_t total = (size_t)num_tokens * N, want = (total + 255) / 256;
   const int blocks = (int)(want > 8192 ? 8192 : want);
-  if (out_dtype == DT_F32) moe_combine_kernel<float><<<blocks, 256, 0, stream>>>(pair_out, top, weight, N, (float*)out, total);
-  else if (out_dtype == DT_BF16) moe_combine_kernel<bf16><<<blocks, 256, 0, stream>>>(pair_out, top, weight, N, (bf16*)out, total);
+  if (out_dtype == DT_F32) moe_combine_kernel<float><<<blocks, 256, 0, stream>>>(pair_out, top, weight, N, (float*)out, total, pair_weight, (const float*)add);
+  else if (out_dtype == DT_BF16) moe_combine_kernel<bf16><<<blocks, 256, 0, stream>>>(pair_out, top, weight, N, (bf16*)out, total, pair_weight, (const bf16*)add);
   else return AS_BAD_DTYPE;
   return launch_status();
 }

@@ -25,7 +25,9 @@ SIGNATURES = {
     "as_qk_norm_rope_store": ("elementwise", [P, I, P, P, I, P, P, P, P, P, I, I, I, I, I, F, I, I, P]),
     "as_silu_mul": ("elementwise", [P, P, I, I, I, P]),
     "as_rmsnorm_multi": ("elementwise", [P, P, P, P, P, P, I, F, P, P, I, I, I, I, P]),
-    "as_head_norm_store": ("elementwise", [P, I, I, I, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, I, I, P]),
+    "as_head_norm_store": ("elementwise", [P, I, I, I, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, I, I, P, I, P]),
+    "as_gated_add_norm": ("elementwise", [P, P, P, I, I, I, P, F, P, P, I, F, P, I, I, I, I, P, P, P]),
+    "as_relu2": ("elementwise", [P, I, I, I, P, I, I, P]),
     "as_sigmoid_gate_heads": ("elementwise", [P, I, I, I, I, P, I, I, F, P, I, I, I, P]),
     "as_short_conv": ("recurrent", [P, I, I, I, I, P, P, P, I, I, I, P, P, P, P, P, P, P, I, I, I, P]),
     "as_delta_prepare": ("recurrent", [P, I, I, I, I, P, I, I, I, I, P, P, I, P, P, I, P]),
@@ -35,7 +37,9 @@ SIGNATURES = {
     "as_rglru_scan": ("recurrent", [P, P, I, P, I, I, I, P, I, F, P, P, P, P, P, I, P, I, I, I, P]),
     "as_moe_route_table": ("moe", [P, P, I, I, I, I, P, P, P, I, P]),
     "as_moe_gemm": ("moe", [P, I, I, P, I, I, I, P, P, P, I, P, I, P]),
-    "as_moe_combine": ("moe", [P, I, F, I, P, I, I, P]),
+    "as_moe_combine": ("moe", [P, I, F, I, P, I, I, P, P, P]),
+    "as_moe_route_sigmoid": ("moe", [P, P, I, I, I, I, I, P, P, P]),
+    "as_attn_headmix": ("attention_mix", [P, P, P, I, P, I, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P]),
     "as_attn_single_query": ("attention", [P, P, P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),
     "as_attn_decode_mfma": ("attention", [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),
     "as_attn_decode_fresh": ("attention", [P, P, P, I, P, P, F, I, P, P, P, I, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),

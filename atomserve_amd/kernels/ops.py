@@ -1029,10 +1029,11 @@ def rmsnorm_multi(x, weight1, weight2, eps, out1, out2=None, delta1=None, delta2
 
 
 def head_norm_store(proj, q_off, k_off, v_off, num_heads, num_kv_heads, dim, vdim, q_weight, k_weight, eps, slots,
-                    q_out, k_pages, v_pages, store_kv=True) -> None:  # fmt: skip
+                    q_out, k_pages, v_pages, store_kv=True, cos_sin=None) -> None:  # fmt: skip
     """Heads cut out of a wider projection's output proj [T, ld] (queries at column q_off, keys at k_off, both
-    `dim` wide; values at v_off, `vdim` wide): per-head RMS norm of queries and keys (weights [dim], or none), no
-    rotation, and the cache store.  Every head is laid out Dp = q_out.shape[2] >= max(dim, vdim) wide, zero where
+    `dim` wide; values at v_off, `vdim` wide): per-head RMS norm of queries and keys (weights [dim], or none), their
+    rotation where `cos_sin` (fp32 [T, R/2, 2]) is given (the pairs (i, i + R/2) of a head's first R coordinates;
+    values are never turned, so v_off = k_off stores the unturned keys as values), and the cache store.  Every head is laid out Dp = q_out.shape[2] >= max(dim, vdim) wide, zero where
     it has no coordinate: q_out [T, H, Dp], k_pages [pages, KV, bs, Dp], v_pages [pages, KV, Dp, bs]."""
     _check(proj, "proj", (F32, BF16), (None, None))
     T, ld = proj.shape
@@ -1057,9 +1058,135 @@ def head_norm_store(proj, q_off, k_off, v_off, num_heads, num_kv_heads, dim, vdi
         _check(k_pages, "k_pages", proj.dtype, (None, KV, None, Dp))
         bs = k_pages.shape[2]
         _check(v_pages, "v_pages", proj.dtype, (k_pages.shape[0], KV, Dp, bs))
+    R = 0
+    if cos_sin is not None:
+        _check(cos_sin, "cos_sin", F32, (T, None, 2))
+        R = 2 * cos_sin.shape[1]
+        if R > dim or R < 2:
+            raise KernelError(f"head_norm_store: {R} turned coordinates in a head of {dim}")
     call("as_head_norm_store", _ptr(proj), _DT[proj.dtype], ld, q_off, k_off, v_off, H, KV, dim, vdim, Dp,
          _ptr(q_weight), _ptr(k_weight), _DT[w_dtype], float(eps), _ptr(slots) if store_kv else 0, _ptr(q_out),
-         _ptr(k_pages) if store_kv else 0, _ptr(v_pages) if store_kv else 0, bs, int(bool(store_kv)), T, _stream())  # fmt: skip
+         _ptr(k_pages) if store_kv else 0, _ptr(v_pages) if store_kv else 0, bs, int(bool(store_kv)), T,
+         _ptr(cos_sin), R, _stream())  # fmt: skip
+
+
+def gated_add_norm(x, y, gate, gate_off, bias, mult, weight, eps, out, rows=None, update_x=True, other=None,
+                   join=None) -> None:  # fmt: skip
+    """The fp32 stream x [T, n] takes a part's gated, scaled output and is normed, in one kernel:
+    x[s] += mult * sigmoid(gate[s, gate_off:gate_off + n] + bias) * y[s]   (y None: nothing is added)
+    out[r] = x[s] / sqrt(mean(x[s]^2) + eps) * weight                      (weight None: no norm; out fp32 or y's dtype)
+    join[r] = [x[s] | other[s]] in the compute dtype                        (join None: none)
+    with s = rows[r] (or r).  y [T, n] and gate [T, ld] are a part's output and the logits of its gate."""
+    _check(x, "x", F32, (None, None))
+    T, n = x.shape
+    n_out = T
+    if rows is not None:
+        _check(rows, "rows", I32, (None,))
+        n_out = rows.shape[0]
+    dtype = None
+    ld = 0
+    if y is not None:
+        _check(y, "y", (F32, BF16), (T, n))
+        dtype = y.dtype
+        _check(gate, "gate", dtype, (T, None))
+        ld = gate.shape[1]
+        if gate_off < 0 or gate_off + n > ld:
+            raise KernelError("gated_add_norm: the gate lies outside its product's columns")
+    if join is not None:
+        _check(join, "join", (F32, BF16) if dtype is None else dtype, (n_out, 2 * n))
+        _check(other, "other", F32, (T, n))
+        dtype = join.dtype
+    w_dtype = None
+    for name, v in (("weight", weight), ("bias", bias)):
+        if v is not None:
+            _check(v, name, (F32, BF16) if w_dtype is None else w_dtype, (n,))
+            w_dtype = v.dtype
+    if weight is not None:
+        _check(out, "out", (F32, BF16), (n_out, n))
+        if dtype is None:
+            dtype = out.dtype if out.dtype == BF16 else weight.dtype
+    if dtype is None:
+        return  # nothing to add, to norm or to join
+    if w_dtype is None:
+        w_dtype = dtype
+    if dtype == F32 and w_dtype != F32:
+        raise KernelError("gated_add_norm: 32-bit rows need 32-bit gains and biases")
+    out_dtype = out.dtype if weight is not None else dtype
+    call("as_gated_add_norm", _ptr(x), _ptr(y), _ptr(gate), _DT[dtype], ld, gate_off, _ptr(bias), float(mult),
+         _ptr(rows), _ptr(weight), _DT[w_dtype], float(eps), _ptr(out) if weight is not None else 0, _DT[out_dtype],
+         n_out, n, int(bool(update_x)), _ptr(other), _ptr(join), _stream())  # fmt: skip
+
+
+def relu2(a, off, out) -> None:
+    """out[t, i] = max(a[t, off + i], 0)^2 for the out.shape[1] columns of a [T, ld] from `off` on."""
+    _check(a, "a", (F32, BF16), (None, None))
+    T, ld = a.shape
+    _check(out, "out", a.dtype, (T, None))
+    n = out.shape[1]
+    if off < 0 or off + n > ld:
+        raise KernelError("relu2: columns outside the input")
+    call("as_relu2", _ptr(a), _DT[a.dtype], ld, off, _ptr(out), n, T, _stream())
+
+
+# ---- attention with mixed heads ----------------------------------------------------------------------
+
+HEADMIX_KEYS = 64  # key slots of a chunk
+HEADMIX_MAX_LDS = 96 << 10
+
+
+def attn_headmix_tile(num_heads: int, head_dim: int, dtype) -> int:
+    """The most consecutive queries of a row that one workgroup of `attn_headmix` takes (16, 8, 4, 2 or 1):
+    bounded by the accumulators a thread keeps and by LDS; 0: the kernel does not take so many heads."""
+    elt = 4 if dtype == F32 else 2
+    for tile, most in ((16, 4), (8, 8), (4, 16), (2, 32), (1, 32)):
+        if -(-num_heads * head_dim // 256) > most:
+            continue
+        floats = 2 * num_heads * tile * HEADMIX_KEYS + num_heads * num_heads + 3 * tile * num_heads + HEADMIX_KEYS
+        if floats * 4 + 16 + tile * num_heads * head_dim * elt > HEADMIX_MAX_LDS:
+            continue
+        return tile
+    return 0
+
+
+def attn_headmix(q, k_pages, v_pages, items, tile: int, positions, tok_row, block_tables, mix, out, scale: float,
+                 window: int = 0, keep_first: int = 0) -> None:  # fmt: skip
+    """Softmax attention whose heads' scores are mixed before the softmax: s_h = sum_g mix[h, g] * scale * q_g . k
+    (mix fp32 [H, H]; None: no mixing), a query at position i seeing the keys j <= i with i - j < window (0: all)
+    or j < keep_first.  q [T, H, D]; out [T, H, Dout], Dout <= D (heads padded to D with zeros lose the padding);
+    pages as the other attention kernels read them.
+    tile == 1: items [N] int32 are single tokens (positions [T]; tok_row [T] or None where token t is row t);
+    else items [N, 4] = (first token, count <= tile, row, first position)."""
+    _check(q, "q", (F32, BF16), (None, None, None))
+    T, H, D = q.shape
+    _check(out, "out", q.dtype, (T, H, None))
+    Dout = out.shape[2]
+    if not 1 <= Dout <= D:
+        raise KernelError(f"attn_headmix: outputs of {Dout} coordinates from heads of {D}")
+    _check(k_pages, "k_pages", q.dtype, (None, None, None, D))
+    NB, KV, bs, _ = k_pages.shape
+    _check(v_pages, "v_pages", q.dtype, (NB, KV, D, bs))
+    _check(block_tables, "block_tables", I32, (None, None))
+    if H % KV or bs > HEADMIX_KEYS:
+        raise KernelError(f"attn_headmix: {H} heads over {KV} kv heads, pages of {bs} (at most {HEADMIX_KEYS})")
+    if D % (4 if q.dtype == F32 else 8):
+        raise KernelError(f"attn_headmix: heads of {D} are not read 16 bytes at a time")
+    most = attn_headmix_tile(H, D, q.dtype)
+    if not 1 <= tile <= most or tile not in (1, 2, 4, 8, 16):
+        raise KernelError(f"attn_headmix: a tile of {tile} queries (at most {most} for {H} heads of {D})")
+    if tile == 1:
+        _check(items, "items", I32, (None,))
+        _check(positions, "positions", I32, (T,))
+        if tok_row is not None:
+            _check(tok_row, "tok_row", I32, (T,))
+    else:
+        _check(items, "items", I32, (None, 4))
+    if mix is not None:
+        _check(mix, "mix", F32, (H, H))
+    if window < 0 or keep_first < 0:
+        raise KernelError("attn_headmix: a window and a number of kept tokens are not negative")
+    call("as_attn_headmix", _ptr(q), _ptr(k_pages), _ptr(v_pages), _DT[q.dtype], _ptr(items), items.shape[0], tile,
+         _ptr(positions), _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(mix), _ptr(out), H, KV, D,
+         Dout, bs, float(scale), int(window), int(keep_first), _stream())  # fmt: skip
 
 
 def sigmoid_gate_heads(heads, vdim, gate, gate_off, scale, out, out_off) -> None:
@@ -1233,7 +1360,7 @@ MOE_MAX_EXPERTS = 1024
 class ExpertRoute:
     """Where a step's (token, chosen expert) pairs stand once sorted by expert: what the grouped products read."""
 
-    __slots__ = ("order", "tiles", "counts", "max_tiles", "top", "num_tokens")
+    __slots__ = ("order", "tiles", "counts", "max_tiles", "top", "num_tokens", "pair_weight")
 
     def __init__(self, num_tokens: int, top: int, experts: int, device):
         pairs = num_tokens * top
@@ -1242,6 +1369,7 @@ class ExpertRoute:
         self.tiles = torch.empty((self.max_tiles, 3), dtype=I32, device=device)
         self.counts = torch.empty(1, dtype=I32, device=device)
         self.top, self.num_tokens = top, num_tokens
+        self.pair_weight = None  # fp32 [pairs]: what each pair weighs, where a router says (else all weigh alike)
 
 
 def moe_route_table(token_ids, table, experts: int) -> ExpertRoute:
@@ -1257,10 +1385,31 @@ def moe_route_table(token_ids, table, experts: int) -> ExpertRoute:
     return route
 
 
-def moe_gemm(a, w, route: ExpertRoute, out, gated: bool, per_token: bool) -> None:
+def moe_route_sigmoid(h, router, top: int) -> ExpertRoute:
+    """Routes by a router's scores: z = router h in fp32, s = sigmoid(z), a token's `top` experts those with the
+    largest s, weighing s / (their sum + 1e-20).  h [T, K], router [experts, K] of one dtype.  The route carries
+    `pair_weight` fp32 [T * top] for `moe_combine`."""
+    _check(h, "h", (F32, BF16), (None, None))
+    T, K = h.shape
+    _check(router, "router", h.dtype, (None, K))
+    experts = router.shape[0]
+    if not 1 <= top <= experts <= MOE_MAX_EXPERTS:
+        raise KernelError(f"routing chooses up to {MOE_MAX_EXPERTS} experts, not {top} of {experts}")
+    route = ExpertRoute(T, top, experts, h.device)
+    pair_expert = torch.empty(max(T * top, 1), dtype=I32, device=h.device)
+    route.pair_weight = torch.empty(max(T * top, 1), dtype=F32, device=h.device)
+    call("as_moe_route_sigmoid", _ptr(h), _ptr(router), _DT[h.dtype], K, experts, top, T, _ptr(pair_expert),
+         _ptr(route.pair_weight), _stream())  # fmt: skip
+    call("as_moe_route_table", 0, _ptr(pair_expert), 0, top, experts, T, _ptr(route.order), _ptr(route.tiles),
+         _ptr(route.counts), route.max_tiles, _stream())  # fmt: skip
+    return route
+
+
+def moe_gemm(a, w, route: ExpertRoute, out, gated: bool, per_token: bool, activation: str = None) -> None:
     """The product of every pair's input with its expert's matrix, w [experts, N_w, K].  per_token: a [T, K] holds
     a row per token (all of a token's pairs read it), else a row per pair.  gated: N_w = 2 N, out[p] =
-    silu(w[e, :N] a) * (w[e, N:] a); else out[p] = w[e] a.  out [pairs, N]: a's dtype, or fp32."""
+    silu(w[e, :N] a) * (w[e, N:] a); else out[p] = w[e] a, or relu(w[e] a)^2 with activation "relu2".
+    out [pairs, N]: a's dtype, or fp32."""
     _check(a, "a", (F32, BF16), (None, None))
     K = a.shape[1]
     pairs = route.num_tokens * route.top
@@ -1271,15 +1420,24 @@ def moe_gemm(a, w, route: ExpertRoute, out, gated: bool, per_token: bool) -> Non
     if gated and w.shape[1] % 2:
         raise KernelError("moe_gemm: gate and up rows come in equal numbers")
     _check(out, "out", (a.dtype, F32), (pairs, N))
-    if gated and out.dtype != a.dtype:
-        raise KernelError("moe_gemm: the gated product's result has the inputs' dtype")
-    call("as_moe_gemm", _ptr(a), _DT[a.dtype], route.top if per_token else 1, _ptr(w), N, K, int(bool(gated)),
+    if activation not in (None, "relu2") or (gated and activation):
+        raise KernelError(f"moe_gemm: activation {activation!r} (None, or 'relu2' on a product without a gate)")
+    if (gated or activation) and out.dtype != a.dtype:
+        raise KernelError("moe_gemm: the activated product's result has the inputs' dtype")
+    call("as_moe_gemm", _ptr(a), _DT[a.dtype], route.top if per_token else 1, _ptr(w), N, K,
+         2 if activation else int(bool(gated)),
          _ptr(route.order), _ptr(route.tiles), _ptr(route.counts), route.max_tiles, _ptr(out), _DT[out.dtype], _stream())  # fmt: skip
 
 
-def moe_combine(pair_out, top: int, weight: float, out) -> None:
-    """out[t] = sum_j weight * pair_out[t * top + j]; pair_out fp32 [T * top, N]."""
+def moe_combine(pair_out, top: int, weight: float, out, pair_weight=None, add=None) -> None:
+    """out[t] = sum_j weight * pair_weight[t * top + j] * pair_out[t * top + j] + add[t]; pair_out fp32 [T * top, N];
+    pair_weight fp32 [T * top] (None: 1); add [T, N] of out's dtype (None: nothing)."""
     _check(out, "out", (F32, BF16), (None, None))
     T, N = out.shape
     _check(pair_out, "pair_out", F32, (T * top, N))
-    call("as_moe_combine", _ptr(pair_out), top, float(weight), N, _ptr(out), _DT[out.dtype], T, _stream())
+    if pair_weight is not None:
+        _check(pair_weight, "pair_weight", F32, (max(T * top, 1),))
+    if add is not None:
+        _check(add, "add", out.dtype, (T, N))
+    call("as_moe_combine", _ptr(pair_out), top, float(weight), N, _ptr(out), _DT[out.dtype], T, _ptr(pair_weight),
+         _ptr(add), _stream())  # fmt: skip

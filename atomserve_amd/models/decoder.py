@@ -6,7 +6,7 @@ the one hard-wired instance of this loop)."""
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import BuildEnv, WeightDecl, build
+from atomserve_amd.parts.base import BuildEnv, GatedDelta, WeightDecl, build
 from atomserve_amd.parts.plan import ModelPlan
 
 
@@ -21,6 +21,11 @@ class DecoderModel:
                             products=ops.ProductChoices())  # fmt: skip
         self.blocks = [build("arrangement", spec, self.env) for spec in plan.layers]
         self.final_norm = build("norm", plan.final_norm, self.env)
+        self.embed_norm = build("norm", plan.embed_norm, self.env) if plan.embed_norm is not None else None
+        if self.embed_norm is not None and not hasattr(self.embed_norm, "stream"):
+            raise ValueError(f"a norm of kind {plan.embed_norm.kind!r} cannot make the embedding's rows the stream")
+        if any(r.reenter for r in plan.run) and not plan.reentry:
+            raise ValueError("a run re-enters the stream, and the plan names no matrix for it (reentry)")
         for r in plan.run:
             if not 0 <= r.layer < len(self.blocks):
                 raise ValueError(f"run list names layer {r.layer}, the plan has {len(self.blocks)}")
@@ -30,7 +35,8 @@ class DecoderModel:
     @property
     def capturable(self) -> bool:
         """Whether a decode step may be captured and replayed as a graph: every part says it is."""
-        return self.final_norm.capturable and all(self.blocks[r.layer].capturable for r in self.plan.run)
+        return self.final_norm.capturable and all(self.blocks[r.layer].capturable for r in self.plan.run) and \
+            (self.embed_norm is None or self.embed_norm.capturable)  # fmt: skip
 
     # ---- tensors --------------------------------------------------------------------
     def weight_decls(self) -> dict:
@@ -42,6 +48,11 @@ class DecoderModel:
                     decls[f"layers.{i}.{part_name}.{local}"] = decl
         for local, decl in self.final_norm.weight_decls().items():
             decls[f"final_norm.{local}"] = decl
+        if self.embed_norm is not None:
+            for local, decl in self.embed_norm.weight_decls().items():
+                decls[f"embed_norm.{local}"] = decl
+        if p.reentry:
+            decls["reentry.weight"] = WeightDecl((p.hidden_size, 2 * p.hidden_size))
         if not p.tied_head:
             decls["head.weight"] = WeightDecl((p.vocab_size, p.hidden_size))
         return decls
@@ -56,6 +67,9 @@ class DecoderModel:
                 prefix = f"layers.{i}.{part_name}."
                 part.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
         self.final_norm.bind({k[len("final_norm."):]: v for k, v in tensors.items() if k.startswith("final_norm.")})
+        if self.embed_norm is not None:
+            self.embed_norm.bind({k[len("embed_norm."):]: v for k, v in tensors.items() if k.startswith("embed_norm.")})
+        self.reentry = ops.Streamed(tensors["reentry.weight"], self.env.stream_copies) if self.plan.reentry else None
         self._tensors = tensors
 
     @property
@@ -67,7 +81,7 @@ class DecoderModel:
     @property
     def num_stream_copy_bytes(self) -> int:
         """Bytes of the copies in wave order that the parts and the head keep beside the tensors."""
-        owned = [self.head] + [w for block in self.blocks for part in block.parts().values() for w in part.streamed()]
+        owned = [self.head] + ([self.reentry] if self.reentry is not None else []) + [w for block in self.blocks for part in block.parts().values() for w in part.streamed()]
         return sum(w.wave_bytes for w in owned)
 
     # ---- caches ---------------------------------------------------------------------
@@ -113,13 +127,43 @@ class DecoderModel:
         p, dev = self.plan, self.env.device
         x = torch.empty((step.num_tokens, p.hidden_size), dtype=torch.float32, device=dev)
         ops.embed_gather(self.embed_weight, step.token_ids, x, p.embedding_scale)
+        x0 = None
+        if self.embed_norm is not None:
+            x0 = self.embed_norm.stream(x)  # fp32: the stream starts as the norm's result, unrounded
+            # the layers change the stream in place; where runs re-enter with what the embedding gave, that is
+            # kept apart (a first run that re-enters replaces the stream before anything has changed it)
+            x = self.embed_norm.stream(x) if p.reentry and not p.run[0].reenter else x0
+        elif p.reentry:
+            x0 = x if p.run[0].reenter else x.clone()
         delta = None
         for i, r in enumerate(p.run):
+            if r.reenter:
+                x, delta = self._reenter(x, delta, x0), None
             # the norm that the run after this one starts with: this run's last product may add
             # into x and leave that norm pending instead of handing over a delta
             follows = self.blocks[p.run[i + 1].layer].first_norm() if i + 1 < len(p.run) else None
             delta = self.blocks[r.layer].forward(x, delta, step, step.cache_view(p.cache_id(i), r.writes),
                                                  next_norm=follows)  # fmt: skip
+        return self._head(x, delta, step, logits)
+
+    def _reenter(self, x, delta, x0):
+        """The stream after the pending output `delta` has been added, beside x0, through the re-entry matrix:
+        a new fp32 stream W [x ; x0]."""
+        T, hidden = x.shape
+        join = torch.empty((T, 2 * hidden), dtype=self.env.dtype, device=x.device)
+        if isinstance(delta, GatedDelta):
+            ops.gated_add_norm(x, delta.y, delta.gate, delta.gate_off, delta.bias, delta.mult, None, 0.0, None,
+                               other=x0, join=join)  # fmt: skip
+        elif delta is None:
+            ops.gated_add_norm(x, None, None, 0, None, 1.0, None, 0.0, None, other=x0, join=join)
+        else:
+            raise ValueError("a run re-enters the stream after a layer that leaves a gated output, or none")
+        out = torch.empty((T, hidden), dtype=torch.float32, device=x.device)
+        ops.gemm(join, self.reentry, out, self.env.products)
+        return out
+
+    def _head(self, x, delta, step, logits):
+        p, dev = self.plan, self.env.device
         n = step.num_logits
         if logits is None:
             logits = torch.empty((n, p.vocab_size), dtype=torch.float32, device=dev)

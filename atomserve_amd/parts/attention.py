@@ -12,7 +12,7 @@ run's cache computes q alone and stores nothing.
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import Mixer, PagedCacheRequest, PendingNorm, SplitSums, WeightDecl, build, register
+from atomserve_amd.parts.base import GatedDelta, Mixer, PagedCacheRequest, PendingNorm, SplitSums, WeightDecl, build, register
 
 # Rows with at most SHORT_ROW new tokens are attended as that many single queries
 # (reference atomserve/runner.py:31-34); longer rows go through the prefill kernel in work items of
@@ -154,3 +154,101 @@ def attend(q, out, step, cache, scale: float, window: int, split) -> None:
 
 
 register("mixer", "attention", Attention)
+
+
+class MixedHeadsAttention(Mixer):
+    """Softmax attention whose heads see each other's scores:
+
+        q = W_q h,  k = W_k h,  v = k as projected (spec.values "keys") or W_v h ("own")
+        q, k turned by the position part (their first R coordinates, pairs (i, i + R/2)); v never
+        raw_g = scale q_g . k_kv(g);  s_h = sum_g M[h, g] raw_g  (spec.mix_heads)
+        j visible from i: j <= i and (i - j < window or j < keep_first)   (window 0: every j <= i)
+        out = W_o [softmax(s_h) v_kv(h)]_h
+
+    q, k (v) and, with spec.out_gate, the logits of the output gate are rows of one input matrix.  A workgroup
+    of the kernel owns all heads of up to `tile` consecutive queries; single tokens are items of one query."""
+
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        s = spec
+        if s.num_heads % s.num_kv_heads:
+            raise ValueError(f"{s.num_heads} query heads do not divide over {s.num_kv_heads} kv heads")
+        if s.values not in ("keys", "own"):
+            raise ValueError(f"values are 'keys' or 'own', not {s.values!r}")
+        self.position = build("position", s.position, env) if s.position is not None else None
+        if self.position is not None and getattr(self.position, "pairs", None) != "half":
+            raise ValueError(f"the kernel turns the pairs (i, i + R/2) by a table of cosines and sines; "
+                             f"{s.position.kind!r} declares {getattr(self.position, 'pairs', None)!r}")  # fmt: skip
+        if s.position is not None and s.position.rotary_dim > s.head_dim:
+            raise ValueError(f"{s.position.rotary_dim} turned coordinates in a head of {s.head_dim}")
+        self.padded_dim = -(-s.head_dim // 8) * 8  # what the kernel reads 16 bytes at a time; the rest is zero
+        self.tile = ops.attn_headmix_tile(s.num_heads, self.padded_dim, env.dtype)
+        if self.tile < 1:
+            raise ValueError(f"{s.num_heads} heads of {s.head_dim} are more than the mixed-heads kernel keeps at once")
+        self.kv_rows = s.num_kv_heads * s.head_dim
+        self.gate_off = s.num_heads * s.head_dim + (1 if s.values == "keys" else 2) * self.kv_rows
+        self.mix_f32 = None
+
+    @property
+    def capturable(self) -> bool:
+        return self.position is None or self.position.capturable
+
+    def weight_decls(self) -> dict:
+        s = self.spec
+        decls = {
+            "in.weight": WeightDecl((self.gate_off + (s.hidden_size if s.out_gate else 0), s.hidden_size)),
+            "o.weight": WeightDecl((s.hidden_size, s.num_heads * s.head_dim)),
+        }
+        if s.mix_heads:
+            decls["mix"] = WeightDecl((s.num_heads, s.num_heads))
+        if s.out_gate:
+            decls["gate_bias"] = WeightDecl((s.hidden_size,), role="vector")
+        return decls
+
+    def bind(self, tensors: dict) -> None:
+        super().bind(tensors)
+        self.win = ops.Streamed(self.in_weight, self.env.stream_copies)
+        self.o = ops.Streamed(self.o_weight, self.env.stream_copies)
+        if self.spec.mix_heads:
+            self.mix_f32 = self.mix.float().contiguous()  # exact: what the file holds in 16 bits widens
+
+    def streamed(self) -> list:
+        return [self.win, self.o]
+
+    def cache_request(self):
+        s = self.spec
+        return PagedCacheRequest(s.num_kv_heads, self.padded_dim, s.window, s.keep_first if s.window > 0 else 0)
+
+    def row_split(self):
+        return (1, self.tile)
+
+    def forward(self, h, step, cache):
+        s, env = self.spec, self.env
+        T, dev = h.shape[0], h.device
+        H, KV, D, Dp = s.num_heads, s.num_kv_heads, s.head_dim, self.padded_dim
+        proj = torch.empty((T, self.in_weight.shape[0]), dtype=env.dtype, device=dev)
+        ops.gemm(h, self.win, proj, env.products)
+        cos_sin = self.position.prepare(step) if self.position is not None else None
+        q = torch.empty((T, H, Dp), dtype=env.dtype, device=dev)
+        k_off = H * D
+        v_off = k_off if s.values == "keys" else k_off + self.kv_rows
+        ops.head_norm_store(proj, 0, k_off, v_off, H, KV, D, D, None, None, 0.0, cache.slots, q, cache.k_pages,
+                            cache.v_pages, store_kv=cache.writes, cos_sin=cos_sin)  # fmt: skip
+        out = torch.empty((T, H, D), dtype=env.dtype, device=dev)
+        args = (cache.block_tables, self.mix_f32, out, s.scale, s.window, s.keep_first)
+        if step.decode_only:  # token t is row t
+            ops.attn_headmix(q, cache.k_pages, cache.v_pages, step.all_tokens, 1, step.positions, None, *args)
+        else:
+            rows = step.split(self.row_split())
+            if rows.num_short_tokens:
+                ops.attn_headmix(q, cache.k_pages, cache.v_pages, rows.short_tokens, 1, step.positions, step.tok_row, *args)
+            if rows.num_long_tiles:
+                ops.attn_headmix(q, cache.k_pages, cache.v_pages, rows.long_tiles, self.tile, None, None, *args)
+        y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=dev)
+        ops.gemm(out.view(T, H * D), self.o, y, env.products)
+        if s.out_gate:
+            return GatedDelta(y, proj, self.gate_off, self.gate_bias)
+        return y
+
+
+register("mixer", "mixed_heads_attention", MixedHeadsAttention)

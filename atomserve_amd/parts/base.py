@@ -47,6 +47,7 @@ class PagedCacheRequest:
     num_kv_heads: int
     head_dim: int
     window: int = 0  # 0: all keys are kept; > 0: pages wholly behind the window are given back
+    keep_first: int = 0  # with a window: the sequence's first tokens that stay visible; their pages are never given back
 
 
 @dataclass(frozen=True)
@@ -137,6 +138,18 @@ class DeltaSum:
         self.parts = tuple(p for p in parts if p is not None)
 
 
+class GatedDelta:
+    """A part's output `y` [T, hidden] still to be added into the stream as mult * sigmoid(gate + bias) * y, the
+    gate's logits being columns gate_off.. of `gate` [T, ld] (a wider product of the part's own): a norm that says
+    `takes_gated_delta` adds it in fp32 on its way."""
+
+    def __init__(self, y, gate, gate_off: int, bias, mult: float = 1.0):
+        self.y, self.gate, self.gate_off, self.bias, self.mult = y, gate, gate_off, bias, mult
+
+    def scaled(self, factor: float) -> "GatedDelta":
+        return GatedDelta(self.y, self.gate, self.gate_off, self.bias, self.mult * factor)
+
+
 class Mixer(Part):
     # Two optional shortcuts an arrangement may take with a part that declares them:
     # takes_pending_norm: `h` may arrive as a PendingNorm instead of normalised rows;
@@ -175,6 +188,7 @@ class FeedForward(Part):
 
 class Norm(Part):
     takes_split_sums = False  # whether `forward` accepts a SplitSums as `delta`
+    takes_gated_delta = False  # whether `forward` accepts a GatedDelta as `delta`
 
     def forward(self, x, delta=None, rows=None, update_residual=True) -> torch.Tensor:
         raise NotImplementedError

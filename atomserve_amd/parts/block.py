@@ -2,6 +2,7 @@
 
 "prenorm":    x += mixer(norm(x));  x += ffn(norm(x))   (reference atomserve/model.py:378-382)
 "two_norms":  x += mixer(norm1(x)) + ffn(norm2(x)), both parts reading the same x through a norm each
+"gated_prenorm": x += m g1(h) * mixer(h), h = norm(x);  x += m g2(h) * ffn(h), h = norm(x), with sigmoid gates g
 
 The residual stream `x` is fp32 in both precisions.  A part's output is not added at
 once: it travels as the pending `delta` to the next norm, whose kernel adds it into
@@ -10,7 +11,7 @@ products around them instead: a part's last product adds into `x` and leaves the
 pending (`Norm.absorb`), and the next part's first product finishes it (`PendingNorm`).
 """
 
-from atomserve_amd.parts.base import Arrangement, DeltaSum, PendingNorm, build, register
+from atomserve_amd.parts.base import Arrangement, DeltaSum, GatedDelta, PendingNorm, build, register
 
 
 class PreNormBlock(Arrangement):
@@ -88,3 +89,46 @@ class TwoNormsBlock(Arrangement):
 
 
 register("arrangement", "two_norms", TwoNormsBlock)
+
+
+class GatedPreNormBlock(Arrangement):
+    """x += m * sigmoid(G h + b) * part(h), h = norm(x), for the mixer and then for the feed-forward (spec.ffn
+    None: the mixer alone); m = spec.residual_scale.  The gate reads what the part reads, so its logits are rows
+    of the part's own input product (parts built with `out_gate` return a `GatedDelta`); the sigmoid, the
+    product with the part's output and the sum into the fp32 stream happen in the kernel of the norm that follows."""
+
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        self.mixer_norm = build("norm", spec.mixer_norm, env)
+        self.mixer = build("mixer", spec.mixer, env)
+        self.ffn_norm = self.ffn = None
+        if spec.ffn is not None:
+            self.ffn_norm = build("norm", spec.ffn_norm, env)
+            self.ffn = build("feed_forward", spec.ffn, env)
+        for name, part in (("mixer", spec.mixer), ("feed-forward", spec.ffn)):
+            if part is not None and not getattr(part, "out_gate", False):
+                raise ValueError(f"a layer with gated residual sums needs a {name} that computes its output gate (out_gate)")
+        for norm in (self.mixer_norm, self.ffn_norm):
+            if norm is not None and not norm.takes_gated_delta:
+                raise ValueError(f"a norm of kind {norm.spec.kind!r} does not add gated outputs into the stream")
+
+    def parts(self) -> dict:
+        parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        if self.ffn is not None:
+            parts.update(ffn_norm=self.ffn_norm, ffn=self.ffn)
+        return parts
+
+    def first_norm(self):
+        return None  # the layer before hands over its output, not a norm left pending in a product
+
+    def forward(self, x, delta, step, cache, next_norm=None):
+        if isinstance(delta, (PendingNorm, DeltaSum)):
+            raise ValueError("a layer with gated residual sums takes a pending output, gated or plain")
+        m = self.spec.residual_scale
+        delta = self.mixer.forward(self.mixer_norm.forward(x, delta), step, cache).scaled(m)
+        if self.ffn is None:
+            return delta
+        return self.ffn.forward(self.ffn_norm.forward(x, delta), step).scaled(m)
+
+
+register("arrangement", "gated_prenorm", GatedPreNormBlock)

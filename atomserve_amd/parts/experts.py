@@ -3,13 +3,14 @@ feed-forwards, down_e(act(gate_e h) * (up_e h)), and their outputs are added wit
 
 Which experts a token uses is found on the GPU, so a step never waits for the host and a decode step can
 be replayed as a graph.  `TableExperts` reads them from a table indexed by the token's id (no router of
-its own: every chosen expert weighs 1 / top); another way of choosing is another `route`.
+its own: every chosen expert weighs 1 / top); `RoutedExperts` scores every expert with a router matrix and
+weighs the chosen by their scores; another way of choosing is another `route`.
 """
 
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import FeedForward, WeightDecl, register
+from atomserve_amd.parts.base import FeedForward, GatedDelta, WeightDecl, register
 
 
 class TableExperts(FeedForward):
@@ -64,3 +65,77 @@ class TableExperts(FeedForward):
 
 
 register("feed_forward", "table_experts", TableExperts)
+
+
+class RoutedExperts(FeedForward):
+    """Experts without a gate, chosen by a router:
+
+        s = sigmoid(R h) in fp32; a token's `top` experts are those with the largest s, weighing s / (their sum + 1e-20)
+        expert e: down_e(relu(up_e h)^2);  with spec.shared_size one more such expert runs for every token and is added
+
+    The shared expert's up rows and, with spec.out_gate, the logits of the output gate are rows of one matrix."""
+
+    capturable = True
+
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        if spec.activation != "relu2":
+            raise ValueError(f"activation {spec.activation!r} has no kernel in experts without a gate (only 'relu2')")
+        if spec.score != "sigmoid":
+            raise ValueError(f"a router scores by 'sigmoid', not by {spec.score!r}")
+        if not 1 <= spec.top <= spec.num_experts <= ops.MOE_MAX_EXPERTS:
+            raise ValueError(f"{spec.top} of {spec.num_experts} experts (at most {ops.MOE_MAX_EXPERTS}) cannot be chosen")
+        self.side_rows = spec.shared_size + (spec.hidden_size if spec.out_gate else 0)
+
+    def weight_decls(self) -> dict:
+        s = self.spec
+        decls = {
+            "router.weight": WeightDecl((s.num_experts, s.hidden_size)),
+            "up.weight": WeightDecl((s.num_experts, s.intermediate_size, s.hidden_size)),
+            "down.weight": WeightDecl((s.num_experts, s.hidden_size, s.intermediate_size)),
+        }
+        if self.side_rows:
+            decls["side.weight"] = WeightDecl((self.side_rows, s.hidden_size))
+        if s.shared_size:
+            decls["shared_down.weight"] = WeightDecl((s.hidden_size, s.shared_size))
+        if s.out_gate:
+            decls["gate_bias"] = WeightDecl((s.hidden_size,), role="vector")
+        return decls
+
+    def bind(self, tensors: dict) -> None:
+        super().bind(tensors)
+        self.side = self.shared_down = None
+        if self.side_rows:
+            self.side = ops.Streamed(self.side_weight, self.env.stream_copies)
+        if self.spec.shared_size:
+            self.shared_down = ops.Streamed(self.shared_down_weight, self.env.stream_copies)
+
+    def streamed(self) -> list:
+        return [w for w in (self.side, self.shared_down) if w is not None]
+
+    def forward(self, h, step):
+        s, env = self.spec, self.env
+        T, dev = h.shape[0], h.device
+        route = ops.moe_route_sigmoid(h, self.router_weight, s.top)
+        pairs = T * s.top
+        act = torch.empty((pairs, s.intermediate_size), dtype=env.dtype, device=dev)
+        ops.moe_gemm(h, self.up_weight, route, act, gated=False, per_token=True, activation=s.activation)
+        each = torch.empty((pairs, s.hidden_size), dtype=torch.float32, device=dev)
+        ops.moe_gemm(act, self.down_weight, route, each, gated=False, per_token=False)
+        side = shared = None
+        if self.side is not None:
+            side = torch.empty((T, self.side_rows), dtype=env.dtype, device=dev)
+            ops.gemm(h, self.side, side, env.products)
+        if s.shared_size:
+            a = torch.empty((T, s.shared_size), dtype=env.dtype, device=dev)
+            ops.relu2(side, 0, a)
+            shared = torch.empty((T, s.hidden_size), dtype=env.dtype, device=dev)
+            ops.gemm(a, self.shared_down, shared, env.products)
+        y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=dev)
+        ops.moe_combine(each, s.top, 1.0, y, pair_weight=route.pair_weight, add=shared)
+        if s.out_gate:
+            return GatedDelta(y, side, s.shared_size, self.gate_bias)
+        return y
+
+
+register("feed_forward", "routed_experts", RoutedExperts)

@@ -6,7 +6,7 @@ pre-norm layer is fused into the same kernel: the fp32 residual stream `x` recei
 import torch
 
 from atomserve_amd.kernels import ops
-from atomserve_amd.parts.base import DeltaSum, Norm, PendingNorm, SplitSums, WeightDecl, register
+from atomserve_amd.parts.base import DeltaSum, GatedDelta, Norm, PendingNorm, SplitSums, WeightDecl, register
 
 
 class PendingRMSNorm(PendingNorm):
@@ -30,6 +30,7 @@ class PendingRMSNorm(PendingNorm):
 class RMSNorm(Norm):
     capturable = True
     takes_split_sums = True
+    takes_gated_delta = True
 
     def weight_decls(self) -> dict:
         return {"weight": WeightDecl((self.spec.size,), role="vector")}
@@ -53,7 +54,10 @@ class RMSNorm(Norm):
         rows: int32 row selection, or None for all rows.  Returns [rows, size], compute dtype."""
         n_out = x.shape[0] if rows is None else rows.shape[0]
         out = torch.empty((n_out, self.spec.size), dtype=self.env.dtype, device=x.device)
-        if isinstance(delta, DeltaSum):
+        if isinstance(delta, GatedDelta):
+            ops.gated_add_norm(x, delta.y, delta.gate, delta.gate_off, delta.bias, delta.mult, self.weight,
+                               self.spec.eps, out, rows=rows, update_x=update_residual)  # fmt: skip
+        elif isinstance(delta, DeltaSum):
             self.with_sibling(None, x, delta, rows, update_residual, out)
         elif isinstance(delta, SplitSums):
             ops.rmsnorm(x, self.weight, self.spec.eps, out, rows=rows, update_x=update_residual, split_sums=delta.sums)
@@ -61,6 +65,13 @@ class RMSNorm(Norm):
             ops.rmsnorm(x, self.weight, self.spec.eps, out, delta=delta, rows=rows, update_x=update_residual)
         return out
 
+
+    def stream(self, x) -> torch.Tensor:
+        """The norm of the fp32 rows x as a new fp32 tensor: for a norm whose result is itself a residual stream
+        (a norm of the embedding), which is never rounded to the compute dtype."""
+        out = torch.empty_like(x)
+        ops.gated_add_norm(x, None, None, 0, None, 1.0, self.weight, self.spec.eps, out, update_x=False)
+        return out
 
     def with_sibling(self, other, x, delta=None, rows=None, update_residual=True, out=None):
         """This norm and `other` (an RMSNorm of the same size and eps, or None) of the same stream in one

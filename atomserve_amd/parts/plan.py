@@ -43,6 +43,28 @@ class AttentionSpec:
 
 
 @dataclass(frozen=True)
+class MixedHeadsAttentionSpec:
+    """Grouped-query softmax attention whose heads' scores are mixed by a matrix [heads, heads] before the
+    softmax (`mix_heads`), over a window that keeps the sequence's first `keep_first` tokens visible
+    (window 0: all keys).  `values` "keys": there is no value projection, a key as projected (before its
+    rotation) is also the value; "own": values have a projection of their own.  `out_gate`: the part also
+    computes sigmoid-gate logits [hidden] of its input (with a bias) for whoever adds its output to the stream."""
+
+    kind: str  # "mixed_heads_attention"
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    scale: float
+    position: Optional[RotarySpec]
+    window: int = 0
+    keep_first: int = 0
+    mix_heads: bool = True
+    values: str = "keys"
+    out_gate: bool = False
+
+
+@dataclass(frozen=True)
 class GatedMLPSpec:
     """Dense gated feed-forward: down(act(gate(x)) * up(x))."""
 
@@ -130,17 +152,38 @@ class TableExpertsSpec:
 
 
 @dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """Experts chosen by a router: scores = `score`(router h) in fp32, the `top` largest are chosen and weigh
+    their scores divided by the chosen scores' sum (+ 1e-20).  An expert is down(act(up h)) without a gate
+    (`activation` "relu2": relu squared).  shared_size > 0: one more expert of that width runs for every token and
+    is added.  `out_gate` as for `MixedHeadsAttentionSpec`."""
+
+    kind: str  # "routed_experts"
+    hidden_size: int
+    intermediate_size: int
+    num_experts: int
+    top: int
+    activation: str  # "relu2"
+    score: str = "sigmoid"
+    shared_size: int = 0
+    out_gate: bool = False
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: a mixer and a feed-forward with their norms, and how they are arranged.
     arrangement "prenorm": x += mixer(norm(x)); x += ffn(norm(x)).
     arrangement "two_norms": x += mixer(mixer_norm(x)) + ffn(ffn_norm(x)), both of the same x
-    (ffn and ffn_norm None: the mixer alone)."""
+    (ffn and ffn_norm None: the mixer alone).
+    arrangement "gated_prenorm": x += m g(h) * mixer(h), h = norm(x); then the same with the feed-forward (or
+    none): m = residual_scale, g the sigmoid gate whose logits the part computes from its input (`out_gate`)."""
 
     arrangement: str
     mixer: Any
     mixer_norm: NormSpec
     ffn: Any
     ffn_norm: Optional[NormSpec]
+    residual_scale: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -151,11 +194,14 @@ class Run:
            the run's index).  Two runs with the same id share one cache.
     writes: whether this run stores what it computes into that cache; a run that only
            reads another run's cache sets this to False.
+    reenter: before this run the stream is replaced by reentry [x ; x0], x0 being what the embedding (and
+           its norm) put into the stream; the plan then names `reentry`.
     """
 
     layer: int
     cache: Optional[int] = None
     writes: bool = True
+    reenter: bool = False
 
 
 @dataclass(frozen=True)
@@ -170,6 +216,8 @@ class ModelPlan:
     embedding_scale: float = 1.0  # multiplies the embedding rows as they enter the stream
     logit_scale: float = 1.0  # multiplies the head's output
     logit_softcap: float = 0.0  # > 0: logits = cap * tanh(logits / cap), after the scale
+    embed_norm: Optional[NormSpec] = None  # a norm of the embedding rows before they become the stream
+    reentry: bool = False  # a matrix [hidden, 2 hidden] through which runs marked `reenter` take [x ; x0]
 
     def cache_id(self, run_index: int) -> int:
         r = self.run[run_index]

@@ -1,7 +1,7 @@
 """Random weights from a configuration and a seed, as a model folder or in memory.
 
 One seeded generator draws every tensor in the order the architecture lists them:
-matrices and biases N(0, std), gains 1 + N(0, gain_std), logarithms of rates N(0, 0.5), tables
+matrices and biases N(0, std), gains 1 + N(0, gain_std), logarithms of rates N(0, 0.5), mixing matrices I + N(0, 0.2), tables
 of experts as rows of distinct expert numbers.  Values are drawn in fp32 and rounded
 to the storage dtype, so a bfloat16 folder read back in float32 holds the same numbers.
 """
@@ -30,6 +30,8 @@ def random_checkpoint(arch, config, seed: int, dtype=torch.bfloat16, device="cpu
             t = t.mul_(gain_std).add_(1.0)
         elif role == "log_rate":
             t = t.mul_(0.5)
+        elif role == "near_identity":  # a square matrix that mixes: the identity and a fifth of it in noise
+            t = t.mul_(0.2).add_(torch.eye(shape[0], device=device))
         else:
             t = t.mul_(std)
         out[name] = t.to(dtype)
