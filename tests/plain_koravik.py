@@ -48,24 +48,33 @@ def visible(T, size, keep_first):
     return (j <= i) & ((i - j < size) | (j < keep_first))
 
 
+def mixed_softmax_attention(q, k, v, talk, scale, size, keep_first):
+    """q [T, H, D], k, v [T, G, D] (positions 0..T-1) -> [T, H, D]: every head's scores are sums of all heads'
+    scores weighed by a row of `talk` [H, H] (None: its own only), then masked and softmaxed."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    kh = k.repeat_interleave(H // G, dim=1)  # head h reads kv head h // (H / G)
+    vh = v.repeat_interleave(H // G, dim=1)
+    s = torch.einsum("ihd,jhd->hij", q, kh) * scale
+    if talk is not None:
+        s = torch.einsum("hg,gij->hij", talk.to(s.dtype), s)
+    s = s.masked_fill(~visible(T, size, keep_first)[None], -math.inf)
+    return torch.einsum("hij,jhd->ihd", torch.softmax(s, dim=-1), vh)
+
+
 def attention(h, w, p, m, round_to=_id):
     """h [T, width]; m: the mixer's configuration; p: the tensors' prefix ('l3.mix.')."""
     T = h.shape[0]
     H, G, D = m["heads"], m["kv_heads"], m["dim"]
     q = round_to(h @ w[p + "q"].T).view(T, H, D)
     k = round_to(h @ w[p + "k"].T).view(T, G, D)
-    v = k
+    v = k  # the keys as projected are the values
     pos = torch.arange(T)
-    q = round_to(turn_half(q, pos, m["rot"]["dims"], m["rot"]["base"]))
-    k = round_to(turn_half(k, pos, m["rot"]["dims"], m["rot"]["base"]))
-    kh = k.repeat_interleave(H // G, dim=1)  # head h reads kv head h // (H / G)
-    vh = v.repeat_interleave(H // G, dim=1)
-    s = torch.einsum("ihd,jhd->hij", q, kh) * m["scale"]
-    s = torch.einsum("hg,gij->hij", w[p + "talk"].to(s.dtype), s)
-    s = s.masked_fill(~visible(T, m["mask"]["size"], m["mask"]["keep_first"])[None], -math.inf)
-    a = torch.softmax(s, dim=-1)
-    o = round_to(torch.einsum("hij,jhd->ihd", a, vh)).reshape(T, H * D)
-    return round_to(o @ w[p + "o"].T)
+    if m["rot"]["dims"]:
+        q = round_to(turn_half(q, pos, m["rot"]["dims"], m["rot"]["base"]))
+        k = round_to(turn_half(k, pos, m["rot"]["dims"], m["rot"]["base"]))
+    o = mixed_softmax_attention(q, k, v, w[p + "talk"], m["scale"], m["mask"]["size"], m["mask"].get("keep_first", 0))
+    return round_to(round_to(o).reshape(T, H * D) @ w[p + "o"].T)
 
 
 def expert(h, up, down, round_to=_id):
@@ -81,9 +90,12 @@ def route(h, router, top):
     return chosen, picked / (picked.sum(-1, keepdim=True) + 1e-20)
 
 
-def experts(h, w, p, f, round_to=_id):
+def experts(h, w, p, f, round_to=_id, routes=None):
+    """routes: a list that receives (scores of all experts, chosen) per call, for tests that look at margins."""
     T = h.shape[0]
     chosen, weights = route(h, w[p + "router"], f["router"]["top"])
+    if routes is not None:
+        routes.append((torch.sigmoid(h @ w[p + "router"].T), chosen))
     out = torch.zeros_like(h)
     for t in range(T):
         for e, a in zip(chosen[t].tolist(), weights[t]):
@@ -117,6 +129,12 @@ def run_order(cfg):
     for _ in range(times):
         order += [(i, i == a) for i in range(a, b)]
     return order + [(i, False) for i in range(b, n)]
+
+
+def logits(cfg, w, tokens, rounded=False):
+    """As the other plain models are called: float64 weights from `w`, logits as float32."""
+    wd = {k: v.double() for k, v in w.items()}
+    return forward(tokens, cfg, wd, round_to=bf16_round if rounded else _id).float()
 
 
 def forward(tokens, cfg, w, round_to=_id, layers_out=None):
