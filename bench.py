@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sizes 8b|0.6b|32b] [--batch B] [--context S]
     python bench.py --workload mixed --sizes 0.6b      (a continuous batch through the scheduler)
     python bench.py --design dozusun [--widths 1024,2048,4096]   (Dozusun layers beside Qwen3 layers of equal size)
+    python bench.py --design koravik [--widths 1024,2048,4096]   (Koravik layers beside Qwen3 layers of equal size)
 
 A step is one decode step of the engine (scheduler, one pass over the GPU, sampling).
 Prints ONE JSON line: decoded tokens per second at batch 8 with 2,048-token contexts,
@@ -75,11 +76,13 @@ def parse_args():
                         "(half of them share their first 32), chunks of 512, 128 tokens decoded each, through the "
                         "scheduler from submission to the last token")  # fmt: skip
     p.add_argument("--chunk-budget", type=int, default=512, help="token budget of a step in the mixed workload")
-    p.add_argument("--design", choices=["qwen3", "dozusun"], default="qwen3",
+    p.add_argument("--design", choices=["qwen3", "dozusun", "koravik"], default="qwen3",
                    help="dozusun: prefill and decode throughput of random-weight Dozusun layers (an attention beside a "
                         "gated linear recurrence, gated delta rules, dense and table-routed feed-forwards) at a few "
-                        "widths, beside Qwen3 layers of the same width, heads, depth and vocabulary")  # fmt: skip
-    p.add_argument("--widths", default="1024,2048,4096", help="stream widths of --design dozusun")
+                        "widths, beside Qwen3 layers of the same width, heads, depth and vocabulary; koravik: the same "
+                        "for Koravik layers (attention with mixed heads and kept first tokens, routed experts with a "
+                        "shared one, gated residual sums, a stretch of layers run twice)")  # fmt: skip
+    p.add_argument("--widths", default="1024,2048,4096", help="stream widths of --design dozusun / koravik")
     p.add_argument("--profile", action="store_true",
                    help="also split the host's time of a decode step into schedule / pack / launch / sample / wait / "
                         "update (steps run one at a time meanwhile, none sent ahead), as the reference's "
@@ -181,10 +184,30 @@ def dozusun_config(width: int, layers: int, vocab: int):
                                     "layers": [pair[i % 2] for i in range(layers)]})  # fmt: skip
 
 
+def koravik_config(width: int, layers: int, vocab: int):
+    """Layers as a model of this design of that width would have them: heads of 128, a kv head to four query heads,
+    a window of 1,024 that keeps the first 64 tokens, 16 experts of three quarters of the width (two to a token) beside
+    a shared expert of one and a half times the width (together the inner width of a feed-forward three times the
+    stream's); `layers` runs of layers: two of the layers form a stretch that runs twice."""
+    from atomserve_amd.config.model_config import KoravikConfig
+
+    heads = width // 128
+    mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128**-0.5,
+             "rot": {"dims": 128, "base": 1e6}, "mask": {"size": 1024, "keep_first": 64}}  # fmt: skip
+    mlp = {"kind": "moe", "expert": {"ff": 3 * width // 4}, "router": {"experts": 16, "top": 2}, "shared": {"ff": 3 * width // 2}}
+    distinct = max(3, layers - 2)
+    return KoravikConfig.from_dict({"architecture": "Koravik", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+                                    "residual_mult": 0.7, "logit_scale": 0.5,
+                                    "layers": [{"type": "attention", "mixer": mixer, "mlp": mlp} for _ in range(distinct)],
+                                    "loop": {"start": 1, "stop": 3, "times": 2}})  # fmt: skip
+
+
 def design_comparison(args) -> dict:
     """Prefill of --prefill-tokens tokens and decode at batch 1 and --batch with --context tokens of context, for
-    Dozusun layers and for Qwen3 layers of equal width, heads, depth and vocabulary; random weights, the engine's own
-    entry point (scheduler, captured decode steps, sampling)."""
+    the layers of --design and for Qwen3 layers of equal width, heads, depth and vocabulary; random weights, the
+    engine's own entry point (scheduler, captured decode steps, sampling)."""
+    design = args.design
+    make = {"dozusun": dozusun_config, "koravik": koravik_config}[design]
     import torch
 
     from atomserve_amd.config import EngineConfig, Qwen3Config
@@ -250,16 +273,16 @@ def design_comparison(args) -> dict:
         qwen = Qwen3Config(vocab_size=vocab, hidden_size=width, intermediate_size=3 * width, num_layers=layers,
                            num_heads=heads, num_kv_heads=max(1, heads // 4), head_dim=128, rms_norm_eps=1e-6,
                            rope_theta=1e6, tie_word_embeddings=False, max_position_embeddings=40960)  # fmt: skip
-        sizes[str(width)] = {"dozusun": measure(dozusun_config(width, layers, vocab)), "qwen3": measure(qwen)}
+        sizes[str(width)] = {design: measure(make(width, layers, vocab)), "qwen3": measure(qwen)}
         print(f"width {width}: {json.dumps(sizes[str(width)])}", file=sys.stderr, flush=True)
     widest = sizes[max(sizes, key=int)]
     return {
-        "metric": f"decode tok/s at batch {args.batch}, {context}-token contexts (Dozusun layers of width {max(sizes, key=int)}, random weights)",
-        "value": widest["dozusun"][f"decode_b{args.batch}_tok_s"],
+        "metric": f"decode tok/s at batch {args.batch}, {context}-token contexts ({design.capitalize()} layers of width {max(sizes, key=int)}, random weights)",
+        "value": widest[design][f"decode_b{args.batch}_tok_s"],
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
-        "ms_per_step": widest["dozusun"][f"decode_b{args.batch}_ms"], "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": widest[design][f"decode_b{args.batch}_ms"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": args.dtype, "data": "synthetic token ids, random-init weights",
-        "config": {"model": "Dozusun layers beside Qwen3 layers of equal size", "layers": layers, "vocab": vocab,
+        "config": {"model": f"{design.capitalize()} layers beside Qwen3 layers of equal size", "layers": layers, "vocab": vocab,
                    "global_batch": args.batch, "seq_len": context, "block_size": block, "parallelism": "single GPU",
                    "sampling": "greedy"},
         "sizes": sizes,
@@ -305,7 +328,7 @@ def main() -> int:
     from atomserve_amd.weights.loader import DictSource, bind_checkpoint
     from atomserve_amd.weights.random_init import random_checkpoint
 
-    if args.design == "dozusun":
+    if args.design in ("dozusun", "koravik"):
         print(json.dumps(design_comparison(args)))
         return 0
     device = "cuda:0"

@@ -590,10 +590,17 @@ def test_the_stream_after_every_layer(dtype):
         block.forward = watched
     replay.step([{"id": "a", "tokens": ids, "want": [44]}], ["a"])
     assert len(seen) == len(want) == 7
+    rounded = []
+    if dtype == "bfloat16":
+        plain.forward(ids, raw, {k: v.double() for k, v in weights.items()}, round_to=plain.bf16_round, layers_out=rounded)
     for i, (got, ref) in enumerate(zip(seen, want)):
-        tol = (2e-5 if dtype == "float32" else 4e-2) * float(ref.abs().max())
         rows = (got.double() - ref).abs().max(-1).values
-        # bfloat16: a token whose two best experts score alike may take the other one; such a row stands out alone
-        allowed = 0 if dtype == "float32" else len(ids) // 8
-        assert int((rows > tol).sum()) <= allowed and float(rows.median()) <= tol, (
-            f"run {i}: {int((rows > tol).sum())} rows beyond {tol:.3e}, the worst {float(rows.max()):.3e} of {float(ref.abs().max()):.3e}")  # fmt: skip
+        if dtype == "float32":
+            assert float(rows.max()) <= 2e-5 * float(ref.abs().max()), f"run {i}: {float(rows.max()):.3e} of {float(ref.abs().max()):.3e}"
+            continue
+        # bfloat16: against what rounding the stored activations moves the plain model's own stream after this run
+        # (a token whose two best experts score alike may take the other one, and every later run carries that on)
+        noise = (rounded[i] - ref).abs().max(-1).values
+        assert float(rows.median()) <= 2.0 * float(noise.median()) and float(rows.max()) <= 3.0 * float(noise.max()), (
+            f"run {i}: rows' median {float(rows.median()):.3e} and worst {float(rows.max()):.3e}; the plain model's "
+            f"{float(noise.median()):.3e} and {float(noise.max()):.3e}")  # fmt: skip
