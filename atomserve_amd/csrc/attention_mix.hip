@@ -55,6 +55,7 @@ struct MixArgs {
   int H, KV, D, Dout, bs;  // Dout <= D: the coordinates of a head that the output keeps (the rest is padding)
   float scale;
   int window, keep_first;
+  int single;  // items are single tokens [N], not (first, count, row, first position) [N, 4]
 };
 
 // accumulators of phase 3 per thread: RMAX (head, d) coordinates by TQ queries
@@ -78,22 +79,27 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_kernel(MixArgs a) {
   T* qs = reinterpret_cast<T*>((reinterpret_cast<uintptr_t>(pages + AM_KC) + 15) & ~(uintptr_t)15);  // [TQ][H][D]
 
   const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
-  int first, count, row, p0;
-  if (TQ == 1) {
-    first = a.items[blockIdx.x];
-    count = 1;
-    row = a.tok_row ? a.tok_row[first] : first;
-    p0 = a.positions[first];
+  int item_first, item_count, row, item_p0;
+  if (a.single) {
+    item_first = a.items[blockIdx.x];
+    item_count = 1;
+    row = a.tok_row ? a.tok_row[item_first] : item_first;
+    item_p0 = a.positions[item_first];
   } else {
     const int* it = a.items + 4 * blockIdx.x;
-    first = it[0]; count = it[1]; row = it[2]; p0 = it[3];
+    item_first = it[0]; item_count = it[1]; row = it[2]; item_p0 = it[3];
   }
   const int* table = a.tables + (size_t)row * a.table_width;
   const T* q = reinterpret_cast<const T*>(a.q);
   const T* kp = reinterpret_cast<const T*>(a.k_pages);
   const T* vp = reinterpret_cast<const T*>(a.v_pages);
+  T* out = reinterpret_cast<T*>(a.out);
 
-  // the pages this item can see: those of the kept first tokens that lie before the window's, then the window's
+  // an item of more queries than TQ is taken TQ at a time
+  for (int qb = 0; qb < item_count; qb += TQ) {
+  const int first = item_first + qb, count = min(TQ, item_count - qb), p0 = item_p0 + qb;
+  if (qb) __syncthreads();  // the queries before have been written out of LDS' statistics
+  // the pages these queries can see: those of the kept first tokens that lie before the window's, then the window's
   const int hi = p0 + count - 1;
   const int lo = a.window > 0 ? max(0, p0 - a.window + 1) : 0;
   const int pb0 = lo / bs, pb1 = hi / bs;
@@ -225,7 +231,6 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_kernel(MixArgs a) {
     }
   }
   __syncthreads();
-  T* out = reinterpret_cast<T*>(a.out);
 #pragma unroll
   for (int r = 0; r < RMAX; ++r) {
     const int e = tid + r * AM_THREADS;
@@ -239,6 +244,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_kernel(MixArgs a) {
       out[((size_t)(first + qi) * H + h) * a.Dout + d] = from_f32<T>(l > 0.f ? acc[r][qi] / l : 0.f);
     }
   }
+  }  // the next TQ queries of the item
 }
 
 static size_t headmix_lds_bytes(int H, int D, int tq, int elt) {
@@ -286,10 +292,13 @@ extern "C" int as_attn_headmix(const void* q, const void* k_pages, const void* v
   const int elt = dtype == DT_F32 ? 4 : 2;
   if (D % (16 / elt)) return AS_BAD_SHAPE;  // rows of keys and queries are read 16 bytes at a time
   const int most = as_attn_headmix_tile(H, D, dtype);
-  if (most <= 0 || tile > most || tile <= 0) return AS_BAD_SHAPE;
+  if (most <= 0 || tile <= 0 || tile > 16) return AS_BAD_SHAPE;
   if (tile == 1 && !positions) return AS_BAD_SHAPE;
   MixArgs a{q, k_pages, v_pages, items, positions, tok_row, tables, table_width, mix, out, H, KV, D, Dout, bs, scale,
-            window, keep_first};
+            window, keep_first, tile == 1};
+  int tq = 1;  // queries a workgroup takes at once: the largest power of two within the items' and what fits
+  while (2 * tq <= tile && 2 * tq <= most) tq *= 2;
+  tile = tq;
   const size_t lds = headmix_lds_bytes(H, D, tile, elt);
 #define GO(T)                                                              \
   switch (tile) {                                                          \
@@ -304,4 +313,293 @@ extern "C" int as_attn_headmix(const void* q, const void* k_pages, const void* v
   if (dtype == DT_BF16) { GO(bf16) }
 #undef GO
   return AS_BAD_DTYPE;
+}
+
+// ---- the same on the matrix cores (bf16) ---------------------------------------------------------------
+// Heads of D % 32 == 0 coordinates, H / KV a power of two up to 16, pages of 8, 16, 32 or 64 tokens.  The 16 rows of
+// a matrix tile are (query, head of one kv head's group): TQ = 16 / group consecutive queries of a row, or one
+// token alone (then only `group` rows stand for something).  Per chunk of 64 key slots:
+//   1. scores: per kv head one product [16 rows x D] [D x 16 keys] a wave (a wave owns 16 of the chunk's keys), the keys
+//      straight from the page as the B operand, the queries from LDS; scaled fp32 scores go to LDS per head;
+//   2. mixing, mask and running softmax on the vector unit in fp32: a lane owns a key slot and a wave eight heads
+//      of a query at a time, so a raw score is read once for eight sums; weights go to LDS as bf16;
+//   3. weights times values: per kv head [16 rows x 64 keys] [64 keys x 16 coordinates] a wave and column tile, the
+//      values straight from the transposed page as the B operand, the outputs in registers for all chunks.
+// `splits` workgroups share an item's chunks and leave unnormalised outputs, maxima and sums for the merge kernel.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+#define AMM_TILES 16  // output tiles (kv head, column tile) a wave keeps: KV * ceil(D / 64) at most
+
+__global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a, int tq, int single, int splits,
+                                                                       float* __restrict__ part_o,
+                                                                       float* __restrict__ part_ml) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int H = a.H, KV = a.KV, D = a.D, bs = a.bs, group = H / KV;
+  const int H8 = (H + 7) & ~7, HB = H8 >> 3;
+  float* sraw = reinterpret_cast<float*>(lds_raw);             // [H][tq][64]
+  float* mixT = sraw + (size_t)H * tq * AM_KC;                 // [H][H8]: mixT[g][h] = mix[h][g]
+  float* row_m = mixT + H * H8;
+  float* row_l = row_m + tq * H;
+  float* row_a = row_l + tq * H;
+  int* pages = reinterpret_cast<int*>(row_a + tq * H);         // [64]
+  bf16* pb = reinterpret_cast<bf16*>((reinterpret_cast<uintptr_t>(pages + AM_KC) + 15) & ~(uintptr_t)15);  // [H][tq][64]
+  bf16* qs = pb + (size_t)H * tq * AM_KC;                      // [tq][H][D]
+
+  const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int item = blockIdx.x, split = blockIdx.y;
+  int first, count, row, p0;
+  if (single) {
+    first = a.items[item];
+    count = 1;
+    row = a.tok_row ? a.tok_row[first] : first;
+    p0 = a.positions[first];
+  } else {
+    const int* it = a.items + 4 * item;
+    first = it[0]; count = it[1]; row = it[2]; p0 = it[3];
+  }
+  const int* table = a.tables + (size_t)row * a.table_width;
+  const bf16* q = reinterpret_cast<const bf16*>(a.q);
+  const bf16* kp = reinterpret_cast<const bf16*>(a.k_pages);
+  const bf16* vp = reinterpret_cast<const bf16*>(a.v_pages);
+  const int HD = H * D, rows_used = tq * group;
+
+  const int hi = p0 + count - 1;
+  const int lo = a.window > 0 ? max(0, p0 - a.window + 1) : 0;
+  const int pb0 = lo / bs, pb1 = hi / bs;
+  const int kept = min(a.keep_first, hi + 1);
+  const int pa_end = min((kept + bs - 1) / bs, pb0);
+  const int NP = pa_end + (pb1 - pb0 + 1);
+  const int ppc = AM_KC / bs;
+  const int chunks = (NP + ppc - 1) / ppc;
+  const int cps = (chunks + splits - 1) / splits;
+  const int ch0 = split * cps, ch1 = min(chunks, ch0 + cps);
+
+  for (int i = tid * 8; i < tq * HD; i += AM_THREADS * 8) {  // 16 bytes a thread: D % 8 == 0
+    const int qi = i / HD;
+    bf16x8 v;
+    if (qi < count) v = *reinterpret_cast<const bf16x8*>(q + (size_t)(first + qi) * HD + (i - qi * HD));
+    else
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (bf16)0.f;
+    *reinterpret_cast<bf16x8*>(qs + i) = v;
+  }
+  for (int i = tid; i < H * H8; i += AM_THREADS) {
+    const int g = i / H8, h = i - g * H8;
+    mixT[i] = h < H ? (a.mix ? a.mix[h * H + g] : (h == g ? 1.f : 0.f)) : 0.f;
+  }
+  for (int i = tid; i < tq * H; i += AM_THREADS) { row_m[i] = -INFINITY; row_l[i] = 0.f; row_a[i] = 1.f; }
+
+  const int CT = D >> 4, CTW = (CT + AM_WAVES - 1) / AM_WAVES;  // column tiles of a head, and of a wave at most
+  floatx4 acc[AMM_TILES];
+#pragma unroll
+  for (int t = 0; t < AMM_TILES; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // the rows this lane meets: as an A operand row lr, as results rows 4 lg + r
+  const int a_qi = lr / group, a_g = lr - a_qi * group;
+  const bool a_valid = lr < rows_used;
+
+  for (int ch = ch0; ch < ch1; ++ch) {
+    __syncthreads();
+    const int u = ch * ppc + lane / bs, off = lane % bs;
+    const bool slot_valid = u < NP;
+    const int lp = u < pa_end ? u : pb0 + (u - pa_end);
+    const int jpos = lp * bs + off;
+    if (tid < AM_KC) pages[tid] = slot_valid ? table[lp] : 0;
+    __syncthreads();
+    // ---- phase 1: scores of this wave's 16 keys for every kv head ---------------------------------
+    {
+      const int slot = 16 * wave + lr;
+      const size_t kbase = ((size_t)pages[slot] * KV * bs + slot % bs) * D;
+      for (int c = 0; c < KV; ++c) {
+        const bf16* krow = kp + kbase + (size_t)c * bs * D;
+        const bf16* qrow = qs + ((size_t)a_qi * H + c * group + a_g) * D;
+        floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int d0 = 0; d0 < D; d0 += 32) {
+          const bf16x8 kb = *reinterpret_cast<const bf16x8*>(krow + d0 + lg * 8);
+          bf16x8 qa;
+          if (a_valid) qa = *reinterpret_cast<const bf16x8*>(qrow + d0 + lg * 8);
+          else
+#pragma unroll
+            for (int j = 0; j < 8; ++j) qa[j] = (bf16)0.f;
+          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kb, sc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int rho = 4 * lg + r;
+          if (rho < rows_used) {
+            const int qi = rho / group, g = rho - qi * group;
+            sraw[((size_t)(c * group + g) * tq + qi) * AM_KC + slot] = sc[r] * a.scale;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // ---- phase 2: mixing, mask, running softmax ------------------------------------------------------
+    for (int unit = wave; unit < tq * HB; unit += AM_WAVES) {
+      const int qi = unit / HB, h0 = (unit - qi * HB) * 8;
+      float mixed[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) mixed[j] = 0.f;
+      for (int g = 0; g < H; ++g) {
+        const float r = sraw[((size_t)g * tq + qi) * AM_KC + lane];
+        const float4 t0 = *reinterpret_cast<const float4*>(mixT + g * H8 + h0);
+        const float4 t1 = *reinterpret_cast<const float4*>(mixT + g * H8 + h0 + 4);
+        mixed[0] = fmaf(t0.x, r, mixed[0]); mixed[1] = fmaf(t0.y, r, mixed[1]);
+        mixed[2] = fmaf(t0.z, r, mixed[2]); mixed[3] = fmaf(t0.w, r, mixed[3]);
+        mixed[4] = fmaf(t1.x, r, mixed[4]); mixed[5] = fmaf(t1.y, r, mixed[5]);
+        mixed[6] = fmaf(t1.z, r, mixed[6]); mixed[7] = fmaf(t1.w, r, mixed[7]);
+      }
+      const int ipos = p0 + qi;
+      const bool seen = slot_valid && qi < count && jpos <= ipos &&
+                        (a.window <= 0 || ipos - jpos < a.window || jpos < a.keep_first);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int h = h0 + j;
+        if (h >= H) break;
+        const int rr = qi * H + h;
+        const float sv = seen ? mixed[j] : -INFINITY;
+        const float m_old = row_m[rr];
+        const float m_new = fmaxf(m_old, wave_max(sv));
+        float p = 0.f, alpha = 1.f;
+        if (m_new > -INFINITY) {
+          p = seen ? expf(sv - m_new) : 0.f;
+          alpha = m_old > -INFINITY ? expf(m_old - m_new) : 0.f;
+        }
+        const float sum = wave_sum(p);
+        pb[((size_t)h * tq + qi) * AM_KC + lane] = (bf16)p;
+        if (lane == 0) {
+          row_m[rr] = m_new;
+          row_l[rr] = row_l[rr] * alpha + sum;
+          row_a[rr] = alpha;
+        }
+      }
+    }
+    __syncthreads();
+    // ---- phase 3: weights times values ------------------------------------------------------------------
+#pragma unroll
+    for (int t = 0; t < AMM_TILES; ++t) {
+      if (t >= KV * CTW) break;
+      const int c = t / CTW, ct = wave + AM_WAVES * (t - c * CTW);
+      if (ct >= CT) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int rho = 4 * lg + r;
+        if (rho < rows_used) {
+          const int qi = rho / group, g = rho - qi * group;
+          acc[t][r] *= row_a[qi * H + c * group + g];
+        }
+      }
+      const bf16* prow = pb + ((size_t)(c * group + a_g) * tq + a_qi) * AM_KC;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const int slot0 = ks * 32 + lg * 8;  // eight slots of one page: pages hold a multiple of 8 tokens
+        bf16x8 pa;
+        if (a_valid) pa = *reinterpret_cast<const bf16x8*>(prow + slot0);
+        else
+#pragma unroll
+          for (int j = 0; j < 8; ++j) pa[j] = (bf16)0.f;
+        const bf16x8 vb = *reinterpret_cast<const bf16x8*>(
+            vp + (((size_t)pages[slot0] * KV + c) * D + ct * 16 + lr) * bs + slot0 % bs);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, acc[t], 0, 0, 0);
+      }
+    }
+  }
+  __syncthreads();
+  bf16* out = reinterpret_cast<bf16*>(a.out);
+  const size_t pbase = ((size_t)item * splits + split) * tq;
+#pragma unroll
+  for (int t = 0; t < AMM_TILES; ++t) {
+    if (t >= KV * CTW) break;
+    const int c = t / CTW, ct = wave + AM_WAVES * (t - c * CTW);
+    if (ct >= CT) continue;
+    const int d = ct * 16 + lr;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int rho = 4 * lg + r;
+      if (rho >= rows_used) continue;
+      const int qi = rho / group, h = c * group + (rho - qi * group);
+      if (qi >= count) continue;
+      if (splits == 1) {
+        const float l = row_l[qi * H + h];
+        if (d < a.Dout) out[((size_t)(first + qi) * H + h) * a.Dout + d] = (bf16)(l > 0.f ? acc[t][r] / l : 0.f);
+      } else {
+        part_o[((pbase + qi) * H + h) * D + d] = acc[t][r];
+      }
+    }
+  }
+  if (splits > 1)
+    for (int i = tid; i < tq * H; i += AM_THREADS) {
+      part_ml[(pbase * H + i) * 2] = row_m[i];
+      part_ml[(pbase * H + i) * 2 + 1] = row_l[i];
+    }
+}
+
+// Puts an item's splits together: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s.  A workgroup per item.
+__global__ __launch_bounds__(AM_THREADS) void attn_headmix_merge_kernel(const int* __restrict__ items, int single, int tq,
+                                                                        int splits, const float* __restrict__ part_o,
+                                                                        const float* __restrict__ part_ml,
+                                                                        bf16* __restrict__ out, int H, int D, int Dout) {
+  const int item = blockIdx.x;
+  const int first = single ? items[item] : items[4 * item], count = single ? 1 : items[4 * item + 1];
+  for (int e = threadIdx.x; e < count * H * D; e += AM_THREADS) {
+    const int qi = e / (H * D), h = (e / D) % H, d = e % D;
+    if (d >= Dout) continue;
+    float M = -INFINITY;
+    for (int s = 0; s < splits; ++s) M = fmaxf(M, part_ml[((((size_t)item * splits + s) * tq + qi) * H + h) * 2]);
+    float num = 0.f, den = 0.f;
+    if (M > -INFINITY)
+      for (int s = 0; s < splits; ++s) {
+        const size_t at = (((size_t)item * splits + s) * tq + qi) * H + h;
+        const float m = part_ml[at * 2];
+        if (m == -INFINITY) continue;
+        const float w = expf(m - M);
+        num = fmaf(w, part_o[at * D + d], num);
+        den = fmaf(w, part_ml[at * 2 + 1], den);
+      }
+    out[((size_t)(first + qi) * H + h) * Dout + d] = (bf16)(den > 0.f ? num / den : 0.f);
+  }
+}
+
+static size_t headmix_mfma_lds(int H, int D, int tq) {
+  const int H8 = (H + 7) & ~7;
+  return ((size_t)H * tq * AM_KC + (size_t)H * H8 + 3 * (size_t)tq * H + AM_KC) * 4 + 16 +
+         ((size_t)H * tq * AM_KC + (size_t)tq * H * D) * 2;
+}
+
+// Whether the matrix-core kernel takes these sizes with items of up to `tq` queries (tq * group rows of a tile).
+static bool headmix_mfma_takes(int H, int KV, int D, int bs, int tq) {
+  if (H <= 0 || KV <= 0 || H % KV || H > 64 || tq < 1) return false;
+  const int group = H / KV;
+  if (group * tq > 16) return false;
+  if (D % 32 || D > 256 || KV * ((D + 63) / 64) > AMM_TILES) return false;
+  if (bs % 8 || bs > AM_KC || AM_KC % bs) return false;
+  return headmix_mfma_lds(H, D, tq) <= (size_t)(128 << 10);
+}
+
+// part_o [num_items, splits, tq, H, D] and part_ml [num_items, splits, tq, H, 2] fp32 where splits > 1.
+extern "C" int as_attn_headmix_mfma(const void* q, const void* k_pages, const void* v_pages, const int* items,
+                                    int num_items, int tq, int single, const int* positions, const int* tok_row,
+                                    const int* tables, int table_width, const float* mix, void* out, int H, int KV,
+                                    int D, int Dout, int bs, float scale, int window, int keep_first, int splits,
+                                    float* part_o, float* part_ml, hipStream_t stream) {
+  if (num_items <= 0) return AS_OK;
+  if (single) tq = 1;
+  if (!headmix_mfma_takes(H, KV, D, bs, tq) || table_width <= 0 || window < 0 || keep_first < 0 || Dout <= 0 || Dout > D || splits < 1 ||
+      splits > 65535 || (splits > 1 && (!part_o || !part_ml)) || (single && !positions))
+    return AS_BAD_SHAPE;
+  MixArgs a{q, k_pages, v_pages, items, positions, tok_row, tables, table_width, mix, out, H, KV, D, Dout, bs, scale,
+            window, keep_first, single};
+  const size_t lds = headmix_mfma_lds(H, D, tq);
+  static bool raised = false;
+  if (lds > (size_t)(64 << 10) && !raised) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_headmix_mfma_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10) != hipSuccess)
+      return AS_LAUNCH_FAILED;
+    raised = true;
+  }
+  attn_headmix_mfma_kernel<<<dim3(num_items, splits), AM_THREADS, lds, stream>>>(a, tq, single, splits, part_o, part_ml);
+  if (splits > 1)
+    attn_headmix_merge_kernel<<<num_items, AM_THREADS, 0, stream>>>(items, single, tq, splits, part_o, part_ml,
+                                                                    (bf16*)out, H, D, Dout);
+  return launch_status();
 }

@@ -39,6 +39,7 @@ SIGNATURES = {
     "as_moe_gemm": ("moe", [P, I, I, P, I, I, I, P, P, P, I, P, I, P]),
     "as_moe_combine": ("moe", [P, I, F, I, P, I, I, P, P, P]),
     "as_moe_route_sigmoid": ("moe", [P, P, I, I, I, I, I, P, P, P]),
+    "as_attn_headmix_mfma": ("attention_mix", [P, P, P, P, I, I, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, P, P, P]),
     "as_attn_headmix": ("attention_mix", [P, P, P, I, P, I, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P]),
     "as_attn_single_query": ("attention", [P, P, P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),
     "as_attn_decode_mfma": ("attention", [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),

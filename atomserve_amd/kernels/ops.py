@@ -1148,14 +1148,64 @@ def attn_headmix_tile(num_heads: int, head_dim: int, dtype) -> int:
     return 0
 
 
+HEADMIX_MFMA_MAX_LDS = 128 << 10
+HEADMIX_MFMA_TILES = 16  # output tiles (kv head, 64 coordinates) that a wave of the matrix-core kernel keeps
+HEADMIX_FILL = 2  # workgroups per compute unit up to which an item's keys are cut over several workgroups
+HEADMIX_MAX_SPLITS = 64
+
+
+def _headmix_mfma_lds(H: int, D: int, tq: int) -> int:
+    h8 = -(-H // 8) * 8
+    return (H * tq * HEADMIX_KEYS + H * h8 + 3 * tq * H + HEADMIX_KEYS) * 4 + 16 + (H * tq * HEADMIX_KEYS + tq * H * D) * 2
+
+
+def attn_headmix_mfma_takes(dtype, H: int, KV: int, D: int, block_size: int, tile: int) -> bool:
+    """Whether the matrix-core form of `attn_headmix` takes these sizes with items of up to `tile` queries: bf16,
+    heads of a multiple of 32 coordinates, `tile` queries times the heads of a kv head within a tile's 16 rows,
+    pages of 8, 16, 32 or 64 tokens."""
+    if dtype != BF16 or H < 1 or KV < 1 or H % KV or H > 64 or tile < 1 or (H // KV) * tile > 16:
+        return False
+    if D % 32 or D > 256 or KV * -(-D // 64) > HEADMIX_MFMA_TILES:
+        return False
+    if block_size % 8 or block_size > HEADMIX_KEYS or HEADMIX_KEYS % block_size:
+        return False
+    return _headmix_mfma_lds(H, D, tile) <= HEADMIX_MFMA_MAX_LDS
+
+
+def attn_headmix_rows(num_heads: int, num_kv_heads: int, head_dim: int, dtype) -> int:
+    """How many consecutive queries of a row make a work item of `attn_headmix` for a model of these sizes: what the
+    matrix-core kernel packs into a tile's 16 rows beside the heads of a kv head, where it takes the sizes at all
+    (whatever the pages: the general kernel serves the pages it does not, taking such an item in turns); else what
+    the general kernel takes at once."""
+    if attn_headmix_mfma_takes(dtype, num_heads, num_kv_heads, head_dim, 16, 1):
+        tile = 16
+        while tile > 1 and not attn_headmix_mfma_takes(dtype, num_heads, num_kv_heads, head_dim, 16, tile):
+            tile //= 2
+        return tile
+    return attn_headmix_tile(num_heads, head_dim, dtype)
+
+
+def _headmix_splits(num_items: int, tile: int, window: int, keep_first: int, max_context: int) -> int:
+    """Into how many workgroups an item's keys are cut: one where the items alone fill the GPU, else as many as fill
+    it, each with at least one chunk of 64 keys."""
+    if max_context <= 0:
+        return 1
+    keys = max_context if window <= 0 else min(max_context, window + tile - 1 + keep_first + HEADMIX_KEYS)
+    chunks = -(-keys // HEADMIX_KEYS) + 1
+    want = -(-HEADMIX_FILL * compute_units() // max(1, num_items))
+    return max(1, min(chunks, want, HEADMIX_MAX_SPLITS))
+
+
 def attn_headmix(q, k_pages, v_pages, items, tile: int, positions, tok_row, block_tables, mix, out, scale: float,
-                 window: int = 0, keep_first: int = 0) -> None:  # fmt: skip
+                 window: int = 0, keep_first: int = 0, max_context: int = 0, splits: int = None) -> None:  # fmt: skip
     """Softmax attention whose heads' scores are mixed before the softmax: s_h = sum_g mix[h, g] * scale * q_g . k
     (mix fp32 [H, H]; None: no mixing), a query at position i seeing the keys j <= i with i - j < window (0: all)
     or j < keep_first.  q [T, H, D]; out [T, H, Dout], Dout <= D (heads padded to D with zeros lose the padding);
     pages as the other attention kernels read them.
     tile == 1: items [N] int32 are single tokens (positions [T]; tok_row [T] or None where token t is row t);
-    else items [N, 4] = (first token, count <= tile, row, first position)."""
+    else items [N, 4] = (first token, count <= tile, row, first position).
+    bf16 with sizes that `attn_headmix_mfma_takes` runs on the matrix cores; max_context (a bound on the positions,
+    0: unknown) lets few items' keys be cut over several workgroups (`splits`: forced, for tests)."""
     _check(q, "q", (F32, BF16), (None, None, None))
     T, H, D = q.shape
     _check(out, "out", q.dtype, (T, H, None))
@@ -1170,9 +1220,11 @@ def attn_headmix(q, k_pages, v_pages, items, tile: int, positions, tok_row, bloc
         raise KernelError(f"attn_headmix: {H} heads over {KV} kv heads, pages of {bs} (at most {HEADMIX_KEYS})")
     if D % (4 if q.dtype == F32 else 8):
         raise KernelError(f"attn_headmix: heads of {D} are not read 16 bytes at a time")
-    most = attn_headmix_tile(H, D, q.dtype)
-    if not 1 <= tile <= most or tile not in (1, 2, 4, 8, 16):
-        raise KernelError(f"attn_headmix: a tile of {tile} queries (at most {most} for {H} heads of {D})")
+    if tile not in (1, 2, 4, 8, 16):
+        raise KernelError(f"attn_headmix: a tile of {tile} queries (1, 2, 4, 8 or 16)")
+    mfma = attn_headmix_mfma_takes(q.dtype, H, KV, D, bs, tile)
+    if not mfma and attn_headmix_tile(H, D, q.dtype) < 1:  # (an item of more queries than fit at once is taken in turns)
+        raise KernelError(f"attn_headmix: {H} heads of {D} are more than a workgroup keeps at once")
     if tile == 1:
         _check(items, "items", I32, (None,))
         _check(positions, "positions", I32, (T,))
@@ -1184,6 +1236,18 @@ def attn_headmix(q, k_pages, v_pages, items, tile: int, positions, tok_row, bloc
         _check(mix, "mix", F32, (H, H))
     if window < 0 or keep_first < 0:
         raise KernelError("attn_headmix: a window and a number of kept tokens are not negative")
+    if mfma:
+        N = items.shape[0]
+        if splits is None:
+            splits = _headmix_splits(N, tile, window, keep_first, max_context)
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = torch.empty((N, splits, tile, H, D), dtype=F32, device=q.device)
+            part_ml = torch.empty((N, splits, tile, H, 2), dtype=F32, device=q.device)
+        call("as_attn_headmix_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(items), N, tile, int(tile == 1),
+             _ptr(positions), _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(mix), _ptr(out), H, KV, D,
+             Dout, bs, float(scale), int(window), int(keep_first), int(splits), _ptr(part_o), _ptr(part_ml), _stream())  # fmt: skip
+        return
     call("as_attn_headmix", _ptr(q), _ptr(k_pages), _ptr(v_pages), _DT[q.dtype], _ptr(items), items.shape[0], tile,
          _ptr(positions), _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(mix), _ptr(out), H, KV, D,
          Dout, bs, float(scale), int(window), int(keep_first), _stream())  # fmt: skip

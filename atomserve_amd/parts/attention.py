@@ -182,7 +182,7 @@ class MixedHeadsAttention(Mixer):
         if s.position is not None and s.position.rotary_dim > s.head_dim:
             raise ValueError(f"{s.position.rotary_dim} turned coordinates in a head of {s.head_dim}")
         self.padded_dim = -(-s.head_dim // 8) * 8  # what the kernel reads 16 bytes at a time; the rest is zero
-        self.tile = ops.attn_headmix_tile(s.num_heads, self.padded_dim, env.dtype)
+        self.tile = ops.attn_headmix_rows(s.num_heads, s.num_kv_heads, self.padded_dim, env.dtype)
         if self.tile < 1:
             raise ValueError(f"{s.num_heads} heads of {s.head_dim} are more than the mixed-heads kernel keeps at once")
         self.kv_rows = s.num_kv_heads * s.head_dim
@@ -237,13 +237,16 @@ class MixedHeadsAttention(Mixer):
         out = torch.empty((T, H, D), dtype=env.dtype, device=dev)
         args = (cache.block_tables, self.mix_f32, out, s.scale, s.window, s.keep_first)
         if step.decode_only:  # token t is row t
-            ops.attn_headmix(q, cache.k_pages, cache.v_pages, step.all_tokens, 1, step.positions, None, *args)
+            ops.attn_headmix(q, cache.k_pages, cache.v_pages, step.all_tokens, 1, step.positions, None, *args,
+                             max_context=step.max_context)  # fmt: skip
         else:
             rows = step.split(self.row_split())
             if rows.num_short_tokens:
-                ops.attn_headmix(q, cache.k_pages, cache.v_pages, rows.short_tokens, 1, step.positions, step.tok_row, *args)
+                ops.attn_headmix(q, cache.k_pages, cache.v_pages, rows.short_tokens, 1, step.positions, step.tok_row, *args,
+                                 max_context=rows.max_short_context)  # fmt: skip
             if rows.num_long_tiles:
-                ops.attn_headmix(q, cache.k_pages, cache.v_pages, rows.long_tiles, self.tile, None, None, *args)
+                ops.attn_headmix(q, cache.k_pages, cache.v_pages, rows.long_tiles, self.tile, None, None, *args,
+                                 max_context=step.max_context)  # fmt: skip
         y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=dev)
         ops.gemm(out.view(T, H * D), self.o, y, env.products)
         if s.out_gate:

@@ -267,7 +267,7 @@ def paged(k, v, block_size, gen, dtype, junk=0.0):
     return kp.to(DEV).to(t), vp.to(DEV).to(t), order.to(torch.int32).view(1, n).to(DEV)
 
 
-def attend(q, kp, vp, table, mix, scale, window, keep_first, dtype, tile, singles=()):
+def attend(q, kp, vp, table, mix, scale, window, keep_first, dtype, tile, singles=(), splits=None):
     """The kernel over one sequence whose queries stand at positions 0..L-1: in tiles of `tile` queries, except the
     positions in `singles`, which go as single tokens."""
     from atomserve_amd.kernels import ops
@@ -286,21 +286,27 @@ def attend(q, kp, vp, table, mix, scale, window, keep_first, dtype, tile, single
         at = s + 1
     if singles:
         items = torch.tensor(sorted(singles), dtype=torch.int32, device=DEV)
-        ops.attn_headmix(qd, kp, vp, items, 1, positions, rows, table, mixd, out, scale, window, keep_first)
+        ops.attn_headmix(qd, kp, vp, items, 1, positions, rows, table, mixd, out, scale, window, keep_first,
+                         max_context=L, splits=splits)  # fmt: skip
     if runs and tile > 1:
         ops.attn_headmix(qd, kp, vp, torch.tensor(runs, dtype=torch.int32, device=DEV), tile, None, None, table, mixd,
-                         out, scale, window, keep_first)  # fmt: skip
+                         out, scale, window, keep_first, max_context=L, splits=splits)  # fmt: skip
     elif runs:
         items = torch.tensor([r[0] for r in runs], dtype=torch.int32, device=DEV)
-        ops.attn_headmix(qd, kp, vp, items, 1, positions, rows, table, mixd, out, scale, window, keep_first)
+        ops.attn_headmix(qd, kp, vp, items, 1, positions, rows, table, mixd, out, scale, window, keep_first,
+                         max_context=L, splits=splits)  # fmt: skip
     return out.float().cpu()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 6, 24, 8), (18, 1, 8, 4), (16, 2, 64, 64), (3, 1, 40, 16), (32, 4, 128, 16)])
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 6, 24, 8), (18, 1, 8, 4), (16, 2, 64, 64), (3, 1, 40, 16), (32, 4, 128, 16),
+                                   (8, 2, 32, 8), (4, 4, 64, 32), (16, 1, 32, 16), (4, 4, 256, 16), (32, 8, 128, 4), (5, 5, 96, 16)])
 def test_mixed_heads_attention_kernel(shape, dtype):
     """Random queries, keys and values over pages in a random order, a window of 37 with 5 kept tokens, a window of
-    one, and none: in tiles, as single tokens, and both in one sequence."""
+    one, and none: in tiles, as single tokens, and both in one sequence.  In bfloat16 the shapes with heads of a
+    multiple of 32 run on the matrix cores (one to sixteen query heads to a kv head, so sixteen to one queries a
+    tile), also with an item's keys cut over three workgroups; pages of 4 tokens and the rest run the general kernel,
+    which takes an item of more queries than it keeps at once in turns."""
     from atomserve_amd.kernels import ops
 
     H, G, D, bs = shape
@@ -308,14 +314,19 @@ def test_mixed_heads_attention_kernel(shape, dtype):
     q, k, v = (bf(torch.randn(L, n, D, generator=gen)) for n in (H, G, G))
     mix = bf(torch.eye(H) + 0.4 * torch.randn(H, H, generator=gen))
     kp, vp, table = paged(k, v, bs, gen, dtype, junk=3.0)
-    tile = ops.attn_headmix_tile(H, D, DTYPES[dtype])
+    tile = ops.attn_headmix_rows(H, G, D, DTYPES[dtype])
     assert tile >= 1
+    on_matrix_cores = ops.attn_headmix_mfma_takes(DTYPES[dtype], H, G, D, bs, tile)
+    assert on_matrix_cores == (dtype == "bfloat16" and D % 32 == 0 and bs >= 8 and H // G in (1, 2, 4, 8, 16))
     tol = 2e-5 if dtype == "float32" else 1.5e-2
     for window, keep in ((37, 5), (1, 0), (0, 0), (20, 33)):
         size = window if window else L + 1
         for talk in (mix, None):
             ref = plain.mixed_softmax_attention(q.double(), k.double(), v.double(), talk, D**-0.5, size, keep).float()
-            for name, kwargs in (("tiles", {}), ("single tokens", {"tile": 1}), ("both", {"singles": (0, 7, 8, 64, 149)})):
+            ways = [("tiles", {}), ("single tokens", {"tile": 1}), ("both", {"singles": (0, 7, 8, 64, 149)})]
+            if on_matrix_cores:
+                ways += [("tiles in three splits", {"splits": 3}), ("both in two splits", {"singles": (1, 63, 148), "splits": 2})]
+            for name, kwargs in ways:
                 got = attend(q, kp, vp, table, talk, D**-0.5, window, keep, dtype, kwargs.pop("tile", tile), **kwargs)
                 assert (got - ref).abs().max() <= tol * float(ref.abs().max()), (
                     f"{shape} window {window} keep {keep} {name}: {float((got - ref).abs().max()):.3e}")  # fmt: skip
