@@ -329,12 +329,18 @@ extern "C" int as_attn_headmix(const void* q, const void* k_pages, const void* v
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 #define AMM_TILES 16  // output tiles (kv head, column tile) a wave keeps: KV * ceil(D / 64) at most
+#define AMM_PIECES 32  // 16-byte pieces of keys, and of values, that a lane asks for per chunk: KV * D / 32 at most
+#define AMM_MAX_SPLITS 64
+// A barrier that waits for this wave's LDS accesses only: a fence would also wait for the loads from memory in flight.
+#define AMM_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
+template <int DS>  // a head's coordinates / 32
 __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a, int tq, int single, int splits,
                                                                        float* __restrict__ part_o,
                                                                        float* __restrict__ part_ml) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  const int H = a.H, KV = a.KV, D = a.D, bs = a.bs, group = H / KV;
+  constexpr int D = 32 * DS, CT = 2 * DS, CTW = (CT + AM_WAVES - 1) / AM_WAVES;  // column tiles of a head, and of a wave at most
+  const int H = a.H, KV = a.KV, bs = a.bs, group = H / KV, gshift = __builtin_ctz(group), gmask = group - 1;
   const int H8 = (H + 7) & ~7, HB = H8 >> 3;
   float* sraw = reinterpret_cast<float*>(lds_raw);             // [H][tq][64]
   float* mixT = sraw + (size_t)H * tq * AM_KC;                 // [H][H8]: mixT[g][h] = mix[h][g]
@@ -390,12 +396,11 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
   }
   for (int i = tid; i < tq * H; i += AM_THREADS) { row_m[i] = -INFINITY; row_l[i] = 0.f; row_a[i] = 1.f; }
 
-  const int CT = D >> 4, CTW = (CT + AM_WAVES - 1) / AM_WAVES;  // column tiles of a head, and of a wave at most
   floatx4 acc[AMM_TILES];
 #pragma unroll
   for (int t = 0; t < AMM_TILES; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
   // the rows this lane meets: as an A operand row lr, as results rows 4 lg + r
-  const int a_qi = lr / group, a_g = lr - a_qi * group;
+  const int a_qi = lr >> gshift, a_g = lr & gmask;
   const bool a_valid = lr < rows_used;
 
   for (int ch = ch0; ch < ch1; ++ch) {
@@ -407,33 +412,69 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
     if (tid < AM_KC) pages[tid] = slot_valid ? table[lp] : 0;
     __syncthreads();
     // ---- phase 1: scores of this wave's 16 keys for every kv head ---------------------------------
+    // (kv head, 32 coordinates) pieces of the wave's keys, sixteen at a time: all of them are asked for before the
+    // first product (a wait for memory per sixteen), in batches of 8 so that small models ask for no more than they have
+    const int slot = 16 * wave + lr;
+    const size_t kbase = ((size_t)pages[slot] * KV * bs + slot % bs) * D;
+    const int total = KV * DS;
+    const size_t q_at = a_valid ? ((size_t)a_qi * H + a_g) * D : 0;  // rows that stand for nothing read row 0 (and are not stored)
     {
-      const int slot = 16 * wave + lr;
-      const size_t kbase = ((size_t)pages[slot] * KV * bs + slot % bs) * D;
-      for (int c = 0; c < KV; ++c) {
-        const bf16* krow = kp + kbase + (size_t)c * bs * D;
-        const bf16* qrow = qs + ((size_t)a_qi * H + c * group + a_g) * D;
-        floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
-        for (int d0 = 0; d0 < D; d0 += 32) {
-          const bf16x8 kb = *reinterpret_cast<const bf16x8*>(krow + d0 + lg * 8);
-          bf16x8 qa;
-          if (a_valid) qa = *reinterpret_cast<const bf16x8*>(qrow + d0 + lg * 8);
-          else
+      floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < 8; ++j) qa[j] = (bf16)0.f;
-          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kb, sc, 0, 0, 0);
+      for (int h0 = 0; h0 < AMM_PIECES; h0 += 16) {
+        if (h0 >= total) break;
+        bf16x8 kb[16];
+#pragma unroll
+        for (int f0 = 0; f0 < 16; f0 += 8) {
+          if (h0 + f0 < total) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              const int f = min(h0 + f0 + i, total - 1);
+              const int c = f / DS, d0 = (f - c * DS) * 32;
+              kb[f0 + i] = *reinterpret_cast<const bf16x8*>(kp + kbase + (size_t)c * bs * D + d0 + lg * 8);
+            }
+          }
         }
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int rho = 4 * lg + r;
-          if (rho < rows_used) {
-            const int qi = rho / group, g = rho - qi * group;
-            sraw[((size_t)(c * group + g) * tq + qi) * AM_KC + slot] = sc[r] * a.scale;
+        for (int i = 0; i < 16; ++i) {
+          const int f = h0 + i;
+          if (f < total) {
+            const int c = f / DS, ds = f - c * DS;
+            const bf16x8 qa = *reinterpret_cast<const bf16x8*>(qs + q_at + (size_t)c * group * D + ds * 32 + lg * 8);
+            if (ds == 0) sc = floatx4{0.f, 0.f, 0.f, 0.f};
+            sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kb[i], sc, 0, 0, 0);
+            if (ds == DS - 1) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int rho = 4 * lg + r;
+                if (rho < rows_used) {
+                  const int qi = rho >> gshift, g = rho & gmask;
+                  sraw[((size_t)(c * group + g) * tq + qi) * AM_KC + slot] = sc[r] * a.scale;
+                }
+              }
+            }
           }
         }
       }
     }
-    __syncthreads();
+    // the first sixteen (output tile, 32 keys) pieces of the chunk's values are asked for now and arrive while the
+    // scores are mixed; a piece that stands for nothing loads what another piece loads and multiplies nothing
+    const int vtotal = 2 * KV * CTW;
+    auto value_piece = [&](int f) {
+      const int t = min(f >> 1, KV * CTW - 1), ks = f & 1;
+      const int c = t / CTW, ct = min(wave + AM_WAVES * (t - c * CTW), CT - 1);
+      const int slot0 = ks * 32 + lg * 8;  // eight slots of one page: pages hold a multiple of 8 tokens
+      return *reinterpret_cast<const bf16x8*>(vp + (((size_t)pages[slot0] * KV + c) * D + ct * 16 + lr) * bs + slot0 % bs);
+    };
+    bf16x8 vb0[16];
+#pragma unroll
+    for (int f0 = 0; f0 < 16; f0 += 8) {
+      if (f0 < vtotal) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) vb0[f0 + i] = value_piece(f0 + i);
+      }
+    }
+    AMM_LDS_BARRIER();
     // ---- phase 2: mixing, mask, running softmax ------------------------------------------------------
     for (int unit = wave; unit < tq * HB; unit += AM_WAVES) {
       const int qi = unit / HB, h0 = (unit - qi * HB) * 8;
@@ -452,56 +493,82 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
       const int ipos = p0 + qi;
       const bool seen = slot_valid && qi < count && jpos <= ipos &&
                         (a.window <= 0 || ipos - jpos < a.window || jpos < a.keep_first);
+      // the eight rows' maxima and sums side by side, so that their lane swaps overlap
+      float mx[8], m_old[8], m_new[8], pr[8], sm[8], al[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        mixed[j] = seen ? mixed[j] : -INFINITY;
+        mx[j] = mixed[j];
+        m_old[j] = h0 + j < H ? row_m[qi * H + h0 + j] : -INFINITY;
+      }
+#pragma unroll
+      for (int off = WAVE / 2; off > 0; off >>= 1)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], off, WAVE));
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        m_new[j] = fmaxf(m_old[j], mx[j]);
+        pr[j] = 0.f;
+        al[j] = 1.f;
+        if (m_new[j] > -INFINITY) {
+          pr[j] = seen ? expf(mixed[j] - m_new[j]) : 0.f;
+          al[j] = m_old[j] > -INFINITY ? expf(m_old[j] - m_new[j]) : 0.f;
+        }
+        sm[j] = pr[j];
+      }
+#pragma unroll
+      for (int off = WAVE / 2; off > 0; off >>= 1)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sm[j] += __shfl_xor(sm[j], off, WAVE);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int h = h0 + j;
         if (h >= H) break;
         const int rr = qi * H + h;
-        const float sv = seen ? mixed[j] : -INFINITY;
-        const float m_old = row_m[rr];
-        const float m_new = fmaxf(m_old, wave_max(sv));
-        float p = 0.f, alpha = 1.f;
-        if (m_new > -INFINITY) {
-          p = seen ? expf(sv - m_new) : 0.f;
-          alpha = m_old > -INFINITY ? expf(m_old - m_new) : 0.f;
-        }
-        const float sum = wave_sum(p);
-        pb[((size_t)h * tq + qi) * AM_KC + lane] = (bf16)p;
+        pb[((size_t)h * tq + qi) * AM_KC + lane] = (bf16)pr[j];
         if (lane == 0) {
-          row_m[rr] = m_new;
-          row_l[rr] = row_l[rr] * alpha + sum;
-          row_a[rr] = alpha;
+          row_m[rr] = m_new[j];
+          row_l[rr] = row_l[rr] * al[j] + sm[j];
+          row_a[rr] = al[j];
         }
       }
     }
-    __syncthreads();
+    AMM_LDS_BARRIER();
     // ---- phase 3: weights times values ------------------------------------------------------------------
-#pragma unroll
-    for (int t = 0; t < AMM_TILES; ++t) {
-      if (t >= KV * CTW) break;
+    const size_t p_at = a_valid ? ((size_t)a_g * tq + a_qi) * AM_KC : 0;
+    auto weigh = [&](int f, const bf16x8& vb, floatx4& o) {  // f static: the tile's accumulator is a register
+      const int t = f >> 1, ks = f & 1;
       const int c = t / CTW, ct = wave + AM_WAVES * (t - c * CTW);
-      if (ct >= CT) continue;
+      if (t < KV * CTW && ct < CT) {
+        if (ks == 0) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int rho = 4 * lg + r;
-        if (rho < rows_used) {
-          const int qi = rho / group, g = rho - qi * group;
-          acc[t][r] *= row_a[qi * H + c * group + g];
+          for (int r = 0; r < 4; ++r) {
+            const int rho = 4 * lg + r;
+            if (rho < rows_used) {
+              const int qi = rho >> gshift, g = rho & gmask;
+              o[r] *= row_a[qi * H + c * group + g];
+            }
+          }
+        }
+        const bf16x8 pa = *reinterpret_cast<const bf16x8*>(pb + p_at + (size_t)c * group * tq * AM_KC + ks * 32 + lg * 8);
+        o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o, 0, 0, 0);
+      }
+    };
+    bf16x8 vb1[16];
+    if (vtotal > 16) {  // the other sixteen pieces, in flight while the first are multiplied
+#pragma unroll
+      for (int f0 = 0; f0 < 16; f0 += 8) {
+        if (16 + f0 < vtotal) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) vb1[f0 + i] = value_piece(16 + f0 + i);
         }
       }
-      const bf16* prow = pb + ((size_t)(c * group + a_g) * tq + a_qi) * AM_KC;
+    }
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const int slot0 = ks * 32 + lg * 8;  // eight slots of one page: pages hold a multiple of 8 tokens
-        bf16x8 pa;
-        if (a_valid) pa = *reinterpret_cast<const bf16x8*>(prow + slot0);
-        else
+    for (int f = 0; f < 16; ++f) weigh(f, vb0[f], acc[f >> 1]);
+    if (vtotal > 16) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) pa[j] = (bf16)0.f;
-        const bf16x8 vb = *reinterpret_cast<const bf16x8*>(
-            vp + (((size_t)pages[slot0] * KV + c) * D + ct * 16 + lr) * bs + slot0 % bs);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, acc[t], 0, 0, 0);
-      }
+      for (int f = 16; f < 32; ++f) weigh(f, vb1[f - 16], acc[f >> 1]);
     }
   }
   __syncthreads();
@@ -517,7 +584,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
     for (int r = 0; r < 4; ++r) {
       const int rho = 4 * lg + r;
       if (rho >= rows_used) continue;
-      const int qi = rho / group, h = c * group + (rho - qi * group);
+      const int qi = rho >> gshift, h = c * group + (rho & gmask);
       if (qi >= count) continue;
       if (splits == 1) {
         const float l = row_l[qi * H + h];
@@ -534,29 +601,35 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
     }
 }
 
-// Puts an item's splits together: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s.  A workgroup per item.
-__global__ __launch_bounds__(AM_THREADS) void attn_headmix_merge_kernel(const int* __restrict__ items, int single, int tq,
-                                                                        int splits, const float* __restrict__ part_o,
-                                                                        const float* __restrict__ part_ml,
-                                                                        bf16* __restrict__ out, int H, int D, int Dout) {
-  const int item = blockIdx.x;
+// Puts an item's splits together: out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s.  A workgroup per (item, head):
+// the splits' weights are made once in LDS, then a thread owns a coordinate and its loads do not wait for one another.
+__global__ __launch_bounds__(128) void attn_headmix_merge_kernel(const int* __restrict__ items, int single, int tq,
+                                                                 int splits, const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml,
+                                                                 bf16* __restrict__ out, int H, int D, int Dout) {
+  __shared__ float wts[AMM_MAX_SPLITS];
+  __shared__ float inv_den;
+  const int item = blockIdx.x, h = blockIdx.y;
   const int first = single ? items[item] : items[4 * item], count = single ? 1 : items[4 * item + 1];
-  for (int e = threadIdx.x; e < count * H * D; e += AM_THREADS) {
-    const int qi = e / (H * D), h = (e / D) % H, d = e % D;
-    if (d >= Dout) continue;
-    float M = -INFINITY;
-    for (int s = 0; s < splits; ++s) M = fmaxf(M, part_ml[((((size_t)item * splits + s) * tq + qi) * H + h) * 2]);
-    float num = 0.f, den = 0.f;
-    if (M > -INFINITY)
-      for (int s = 0; s < splits; ++s) {
-        const size_t at = (((size_t)item * splits + s) * tq + qi) * H + h;
-        const float m = part_ml[at * 2];
-        if (m == -INFINITY) continue;
-        const float w = expf(m - M);
-        num = fmaf(w, part_o[at * D + d], num);
-        den = fmaf(w, part_ml[at * 2 + 1], den);
-      }
-    out[((size_t)(first + qi) * H + h) * Dout + d] = (bf16)(den > 0.f ? num / den : 0.f);
+  for (int qi = 0; qi < count; ++qi) {
+    __syncthreads();
+    if (threadIdx.x < WAVE) {  // splits <= 64: one lane each
+      const int s = threadIdx.x;
+      const size_t at = (((size_t)item * splits + min(s, splits - 1)) * tq + qi) * H + h;
+      const float m = s < splits ? part_ml[at * 2] : -INFINITY;
+      const float M = wave_max(m);
+      const float w = (s < splits && m > -INFINITY) ? expf(m - M) : 0.f;
+      const float den = wave_sum(s < splits ? w * part_ml[at * 2 + 1] : 0.f);
+      wts[s] = w;
+      if (s == 0) inv_den = den > 0.f ? 1.0f / den : 0.f;
+    }
+    __syncthreads();
+    for (int d = threadIdx.x; d < Dout; d += blockDim.x) {
+      float num = 0.f;
+      for (int s = 0; s < splits; ++s)
+        num = fmaf(wts[s], part_o[((((size_t)item * splits + s) * tq + qi) * H + h) * D + d], num);
+      out[((size_t)(first + qi) * H + h) * Dout + d] = (bf16)(num * inv_den);
+    }
   }
 }
 
@@ -571,7 +644,7 @@ static bool headmix_mfma_takes(int H, int KV, int D, int bs, int tq) {
   if (H <= 0 || KV <= 0 || H % KV || H > 64 || tq < 1) return false;
   const int group = H / KV;
   if (group * tq > 16) return false;
-  if (D % 32 || D > 256 || KV * ((D + 63) / 64) > AMM_TILES) return false;
+  if (D % 32 || D > 256 || D == 160 || D == 224 || KV * ((D + 63) / 64) > AMM_TILES) return false;
   if (bs % 8 || bs > AM_KC || AM_KC % bs) return false;
   return headmix_mfma_lds(H, D, tq) <= (size_t)(128 << 10);
 }
@@ -585,21 +658,31 @@ extern "C" int as_attn_headmix_mfma(const void* q, const void* k_pages, const vo
   if (num_items <= 0) return AS_OK;
   if (single) tq = 1;
   if (!headmix_mfma_takes(H, KV, D, bs, tq) || table_width <= 0 || window < 0 || keep_first < 0 || Dout <= 0 || Dout > D || splits < 1 ||
-      splits > 65535 || (splits > 1 && (!part_o || !part_ml)) || (single && !positions))
+      splits > AMM_MAX_SPLITS || (splits > 1 && (!part_o || !part_ml)) || (single && !positions))
     return AS_BAD_SHAPE;
   MixArgs a{q, k_pages, v_pages, items, positions, tok_row, tables, table_width, mix, out, H, KV, D, Dout, bs, scale,
             window, keep_first, single};
   const size_t lds = headmix_mfma_lds(H, D, tq);
-  static bool raised = false;
-  if (lds > (size_t)(64 << 10) && !raised) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_headmix_mfma_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10) != hipSuccess)
-      return AS_LAUNCH_FAILED;
-    raised = true;
+#define GO(DS)                                                                                                     \
+  case DS: {                                                                                                       \
+    static bool raised = false; /* a workgroup may ask for more than 64 KB of LDS once the kernel says so */       \
+    if (lds > (size_t)(64 << 10) && !raised) {                                                                     \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_headmix_mfma_kernel<DS>),                        \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10) != hipSuccess)                \
+        return AS_LAUNCH_FAILED;                                                                                   \
+      raised = true;                                                                                               \
+    }                                                                                                              \
+    attn_headmix_mfma_kernel<DS><<<dim3(num_items, splits), AM_THREADS, lds, stream>>>(a, tq, single, splits,      \
+                                                                                       part_o, part_ml);           \
+    break;                                                                                                         \
   }
-  attn_headmix_mfma_kernel<<<dim3(num_items, splits), AM_THREADS, lds, stream>>>(a, tq, single, splits, part_o, part_ml);
+  switch (D / 32) {
+    GO(1) GO(2) GO(3) GO(4) GO(6) GO(8)
+    default: return AS_BAD_SHAPE;
+  }
+#undef GO
   if (splits > 1)
-    attn_headmix_merge_kernel<<<num_items, AM_THREADS, 0, stream>>>(items, single, tq, splits, part_o, part_ml,
-                                                                    (bf16*)out, H, D, Dout);
+    attn_headmix_merge_kernel<<<dim3(num_items, H), 128, 0, stream>>>(items, single, tq, splits, part_o, part_ml,
+                                                                      (bf16*)out, H, D, Dout);
   return launch_status();
 }

@@ -77,27 +77,53 @@ __global__ __launch_bounds__(1024) void moe_route_table_kernel(const int* __rest
 // ---- a router that scores every expert ---------------------------------------------------------------
 // z = router h in fp32 (router [experts, K], h [T, K], both T-typed), s = sigmoid(z); a token's `top` experts are
 // those with the largest s (of equal ones the lower number first); their weights are s / (sum of the chosen + 1e-20).
-// pair_expert, pair_weight [T * top].  A wave per token: every lane walks the width in strides for one expert
-// after the other, the sums meet by lane swaps, the choice runs over LDS.
+// pair_expert, pair_weight [T * top].  A workgroup per token: its waves take the experts in turn, a lane 16 bytes of
+// the router's row and of the token's at a time (the rows stream once, coalesced), the sums meet by lane swaps and the
+// scores in LDS, where the first wave makes the choice.
+template <typename T> struct RoutePiece;
+template <> struct RoutePiece<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ float dot(const float* a, const float* b) {
+    const float4 x = *reinterpret_cast<const float4*>(a), y = *reinterpret_cast<const float4*>(b);
+    return fmaf(x.w, y.w, fmaf(x.z, y.z, fmaf(x.y, y.y, x.x * y.x)));
+  }
+};
+template <> struct RoutePiece<bf16> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ float dot(const bf16* a, const bf16* b) {
+    const bf16x8 x = *reinterpret_cast<const bf16x8*>(a), y = *reinterpret_cast<const bf16x8*>(b);
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s = fmaf((float)x[i], (float)y[i], s);
+    return s;
+  }
+};
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(const T* __restrict__ h, const T* __restrict__ router,
                                                                 int K, int experts, int top, int num_tokens,
                                                                 int* __restrict__ pair_expert,
                                                                 float* __restrict__ pair_weight) {
-  extern __shared__ float scores[];  // [4][experts]
+  extern __shared__ float scores[];  // [experts]
+  constexpr int N = RoutePiece<T>::N;
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
-  const int t = blockIdx.x * 4 + wave;
-  if (t >= num_tokens) return;
-  float* mine = scores + (size_t)wave * experts;
+  const int t = blockIdx.x;
   const T* row = h + (size_t)t * K;
-  for (int e = 0; e < experts; ++e) {
+  const bool whole = K % N == 0;  // rows start on 16 bytes
+  for (int e = wave; e < experts; e += 4) {
     const T* wr = router + (size_t)e * K;
     float z = 0.f;
-    for (int k = lane; k < K; k += WAVE) z = fmaf(to_f32(row[k]), to_f32(wr[k]), z);
+    if (whole) {
+      for (int k = lane * N; k < K; k += WAVE * N) z += RoutePiece<T>::dot(row + k, wr + k);
+    } else {
+      for (int k = lane; k < K; k += WAVE) z = fmaf(to_f32(row[k]), to_f32(wr[k]), z);
+    }
     z = wave_sum(z);
-    if (lane == 0) mine[e] = 1.0f / (1.0f + expf(-z));
+    if (lane == 0) scores[e] = 1.0f / (1.0f + expf(-z));
   }
-  __builtin_amdgcn_wave_barrier();
+  __syncthreads();
+  if (wave) return;
+  float* mine = scores;
   float total = 0.f, my_score = 0.f;
   int my_expert = 0;
   for (int j = 0; j < top; ++j) {
@@ -136,8 +162,8 @@ extern "C" int as_moe_route_sigmoid(const void* h, const void* router, int dtype
                                     int num_tokens, int* pair_expert, float* pair_weight, hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
   if (K <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts) return AS_BAD_SHAPE;
-  const int blocks = (num_tokens + 3) / 4;
-  const size_t lds = (size_t)4 * experts * sizeof(float);
+  const int blocks = num_tokens;
+  const size_t lds = (size_t)experts * sizeof(float);
   if (dtype == DT_F32)
     moe_route_sigmoid_kernel<float><<<blocks, 256, lds, stream>>>((const float*)h, (const float*)router, K, experts, top,
                                                                   num_tokens, pair_expert, pair_weight);

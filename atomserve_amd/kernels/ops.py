@@ -1161,11 +1161,11 @@ def _headmix_mfma_lds(H: int, D: int, tq: int) -> int:
 
 def attn_headmix_mfma_takes(dtype, H: int, KV: int, D: int, block_size: int, tile: int) -> bool:
     """Whether the matrix-core form of `attn_headmix` takes these sizes with items of up to `tile` queries: bf16,
-    heads of a multiple of 32 coordinates, `tile` queries times the heads of a kv head within a tile's 16 rows,
+    heads of 32, 64, 96, 128, 192 or 256 coordinates, `tile` queries times the heads of a kv head within a tile's 16 rows,
     pages of 8, 16, 32 or 64 tokens."""
     if dtype != BF16 or H < 1 or KV < 1 or H % KV or H > 64 or tile < 1 or (H // KV) * tile > 16:
         return False
-    if D % 32 or D > 256 or KV * -(-D // 64) > HEADMIX_MFMA_TILES:
+    if D not in (32, 64, 96, 128, 192, 256) or KV * -(-D // 64) > HEADMIX_MFMA_TILES:
         return False
     if block_size % 8 or block_size > HEADMIX_KEYS or HEADMIX_KEYS % block_size:
         return False
