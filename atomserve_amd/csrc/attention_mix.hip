@@ -481,6 +481,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
       float mixed[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) mixed[j] = 0.f;
+#pragma unroll 4
       for (int g = 0; g < H; ++g) {
         const float r = sraw[((size_t)g * tq + qi) * AM_KC + lane];
         const float4 t0 = *reinterpret_cast<const float4*>(mixT + g * H8 + h0);

@@ -762,7 +762,8 @@ extern "C" int as_gated_add_norm(float* x, const void* y, const void* gate, int 
   if (n <= 0 || (y && (!gate || ld_gate < n || gate_off < 0 || gate_off + n > ld_gate)) || (w && !out) ||
       (join && !other))
     return AS_BAD_SHAPE;
-  const int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : 64);
+  // four values a thread where the row allows it: a decode step's few rows wait for memory, not for arithmetic
+  const int threads = n >= 4096 ? 1024 : (n >= 2048 ? 512 : (n >= 512 ? 256 : 64));
 #define LAUNCH(O, W, NO)                                                                                          \
   gated_add_norm_kernel<O, W, NO><<<n_out, threads, 0, stream>>>(x, (const O*)y, (const O*)gate, ld_gate, gate_off, \
                                                                  (const W*)bias, mult, rows, (const W*)w, eps,      \
