@@ -329,17 +329,18 @@ extern "C" int as_attn_headmix(const void* q, const void* k_pages, const void* v
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 #define AMM_TILES 16  // output tiles (kv head, column tile) a wave keeps: KV * ceil(D / 64) at most
+#define AMM_THREADS 512  // eight waves, two to a SIMD
 #define AMM_PIECES 32  // 16-byte pieces of keys, and of values, that a lane asks for per chunk: KV * D / 32 at most
 #define AMM_MAX_SPLITS 64
 // A barrier that waits for this wave's LDS accesses only: a fence would also wait for the loads from memory in flight.
 #define AMM_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
 template <int DS>  // a head's coordinates / 32
-__global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a, int tq, int single, int splits,
+__global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs a, int tq, int single, int splits,
                                                                        float* __restrict__ part_o,
                                                                        float* __restrict__ part_ml) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  constexpr int D = 32 * DS, CT = 2 * DS, CTW = (CT + AM_WAVES - 1) / AM_WAVES;  // column tiles of a head, and of a wave at most
+  constexpr int D = 32 * DS, CT = 2 * DS, CTW = (CT + 3) / 4;  // column tiles of a head, and of a wave at most
   const int H = a.H, KV = a.KV, bs = a.bs, group = H / KV, gshift = __builtin_ctz(group), gmask = group - 1;
   const int H8 = (H + 7) & ~7, HB = H8 >> 3;
   float* sraw = reinterpret_cast<float*>(lds_raw);             // [H][tq][64]
@@ -351,8 +352,11 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
   bf16* pb = reinterpret_cast<bf16*>((reinterpret_cast<uintptr_t>(pages + AM_KC) + 15) & ~(uintptr_t)15);  // [H][tq][64]
   bf16* qs = pb + (size_t)H * tq * AM_KC;                      // [tq][H][D]
 
-  const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+  // eight waves: wave & 3 says which 16 of a chunk's keys (scores) and which column tiles (values) a wave takes,
+  // wave >> 2 which half of the kv heads (the even or the odd ones); two waves share a SIMD and fill each other's waits
+  const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave8 = tid / WAVE, wave = wave8 & 3, half = wave8 >> 2;
   const int lr = lane & 15, lg = lane >> 4;
+  const int KVh = (KV - half + 1) >> 1;  // kv heads of this wave's half: c = 2 c' + half
   const int item = blockIdx.x, split = blockIdx.y;
   int first, count, row, p0;
   if (single) {
@@ -381,7 +385,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
   const int cps = (chunks + splits - 1) / splits;
   const int ch0 = split * cps, ch1 = min(chunks, ch0 + cps);
 
-  for (int i = tid * 8; i < tq * HD; i += AM_THREADS * 8) {  // 16 bytes a thread: D % 8 == 0
+  for (int i = tid * 8; i < tq * HD; i += AMM_THREADS * 8) {  // 16 bytes a thread: D % 8 == 0
     const int qi = i / HD;
     bf16x8 v;
     if (qi < count) v = *reinterpret_cast<const bf16x8*>(q + (size_t)(first + qi) * HD + (i - qi * HD));
@@ -390,15 +394,15 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
       for (int j = 0; j < 8; ++j) v[j] = (bf16)0.f;
     *reinterpret_cast<bf16x8*>(qs + i) = v;
   }
-  for (int i = tid; i < H * H8; i += AM_THREADS) {
+  for (int i = tid; i < H * H8; i += AMM_THREADS) {
     const int g = i / H8, h = i - g * H8;
     mixT[i] = h < H ? (a.mix ? a.mix[h * H + g] : (h == g ? 1.f : 0.f)) : 0.f;
   }
-  for (int i = tid; i < tq * H; i += AM_THREADS) { row_m[i] = -INFINITY; row_l[i] = 0.f; row_a[i] = 1.f; }
+  for (int i = tid; i < tq * H; i += AMM_THREADS) { row_m[i] = -INFINITY; row_l[i] = 0.f; row_a[i] = 1.f; }
 
-  floatx4 acc[AMM_TILES];
+  floatx4 acc[AMM_TILES / 2];
 #pragma unroll
-  for (int t = 0; t < AMM_TILES; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < AMM_TILES / 2; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
   // the rows this lane meets: as an A operand row lr, as results rows 4 lg + r
   const int a_qi = lr >> gshift, a_g = lr & gmask;
   const bool a_valid = lr < rows_used;
@@ -414,14 +418,18 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
     // ---- phase 1: scores of this wave's 16 keys for every kv head ---------------------------------
     // (kv head, 32 coordinates) pieces of the wave's keys, sixteen at a time: all of them are asked for before the
     // first product (a wait for memory per sixteen), in batches of 8 so that small models ask for no more than they have
-    const int slot = 16 * wave + lr;
+    // what a lane adds to its addresses, hidden from the compiler at every chunk: it would otherwise keep every
+    // piece's address in registers of its own for the whole kernel (a hundred of them) and spill the products' operands
+    int lg8 = lg * 8, lrv = lr;
+    asm volatile("" : "+v"(lg8), "+v"(lrv));
+    const int slot = 16 * wave + lrv;
     const size_t kbase = ((size_t)pages[slot] * KV * bs + slot % bs) * D;
-    const int total = KV * DS;
+    const int total = KVh * DS;
     const size_t q_at = a_valid ? ((size_t)a_qi * H + a_g) * D : 0;  // rows that stand for nothing read row 0 (and are not stored)
     {
       floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int h0 = 0; h0 < AMM_PIECES; h0 += 16) {
+      for (int h0 = 0; h0 < AMM_PIECES / 2; h0 += 16) {
         if (h0 >= total) break;
         bf16x8 kb[16];
 #pragma unroll
@@ -430,8 +438,8 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
               const int f = min(h0 + f0 + i, total - 1);
-              const int c = f / DS, d0 = (f - c * DS) * 32;
-              kb[f0 + i] = *reinterpret_cast<const bf16x8*>(kp + kbase + (size_t)c * bs * D + d0 + lg * 8);
+              const int c = 2 * (f / DS) + half, d0 = (f % DS) * 32;
+              kb[f0 + i] = *reinterpret_cast<const bf16x8*>(kp + kbase + (size_t)c * bs * D + d0 + lg8);
             }
           }
         }
@@ -439,8 +447,8 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
         for (int i = 0; i < 16; ++i) {
           const int f = h0 + i;
           if (f < total) {
-            const int c = f / DS, ds = f - c * DS;
-            const bf16x8 qa = *reinterpret_cast<const bf16x8*>(qs + q_at + (size_t)c * group * D + ds * 32 + lg * 8);
+            const int c = 2 * (f / DS) + half, ds = f % DS;
+            const bf16x8 qa = *reinterpret_cast<const bf16x8*>(qs + q_at + (size_t)c * group * D + ds * 32 + lg8);
             if (ds == 0) sc = floatx4{0.f, 0.f, 0.f, 0.f};
             sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kb[i], sc, 0, 0, 0);
             if (ds == DS - 1) {
@@ -457,26 +465,21 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
         }
       }
     }
-    // the first sixteen (output tile, 32 keys) pieces of the chunk's values are asked for now and arrive while the
+    // the first eight (output tile, 32 keys) pieces of the chunk's values are asked for now and arrive while the
     // scores are mixed; a piece that stands for nothing loads what another piece loads and multiplies nothing
-    const int vtotal = 2 * KV * CTW;
+    const int vtotal = 2 * KVh * CTW;
     auto value_piece = [&](int f) {
-      const int t = min(f >> 1, KV * CTW - 1), ks = f & 1;
-      const int c = t / CTW, ct = min(wave + AM_WAVES * (t - c * CTW), CT - 1);
-      const int slot0 = ks * 32 + lg * 8;  // eight slots of one page: pages hold a multiple of 8 tokens
-      return *reinterpret_cast<const bf16x8*>(vp + (((size_t)pages[slot0] * KV + c) * D + ct * 16 + lr) * bs + slot0 % bs);
+      const int t = min(f >> 1, max(KVh * CTW - 1, 0)), ks = f & 1;
+      const int c = min(2 * (t / CTW) + half, KV - 1), ct = min(wave + 4 * (t % CTW), CT - 1);
+      const int slot0 = ks * 32 + lg8;  // eight slots of one page: pages hold a multiple of 8 tokens
+      return *reinterpret_cast<const bf16x8*>(vp + (((size_t)pages[slot0] * KV + c) * D + ct * 16 + lrv) * bs + slot0 % bs);
     };
-    bf16x8 vb0[16];
+    bf16x8 vb0[8];
 #pragma unroll
-    for (int f0 = 0; f0 < 16; f0 += 8) {
-      if (f0 < vtotal) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) vb0[f0 + i] = value_piece(f0 + i);
-      }
-    }
+    for (int i = 0; i < 8; ++i) vb0[i] = value_piece(i);
     AMM_LDS_BARRIER();
     // ---- phase 2: mixing, mask, running softmax ------------------------------------------------------
-    for (int unit = wave; unit < tq * HB; unit += AM_WAVES) {
+    for (int unit = wave8; unit < tq * HB; unit += 8) {
       const int qi = unit / HB, h0 = (unit - qi * HB) * 8;
       float mixed[8];
 #pragma unroll
@@ -539,8 +542,8 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
     const size_t p_at = a_valid ? ((size_t)a_g * tq + a_qi) * AM_KC : 0;
     auto weigh = [&](int f, const bf16x8& vb, floatx4& o) {  // f static: the tile's accumulator is a register
       const int t = f >> 1, ks = f & 1;
-      const int c = t / CTW, ct = wave + AM_WAVES * (t - c * CTW);
-      if (t < KV * CTW && ct < CT) {
+      const int c = 2 * (t / CTW) + half, ct = wave + 4 * (t % CTW);
+      if (t < KVh * CTW && ct < CT) {
         if (ks == 0) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
@@ -551,34 +554,29 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
             }
           }
         }
-        const bf16x8 pa = *reinterpret_cast<const bf16x8*>(pb + p_at + (size_t)c * group * tq * AM_KC + ks * 32 + lg * 8);
+        const bf16x8 pa = *reinterpret_cast<const bf16x8*>(pb + p_at + (size_t)c * group * tq * AM_KC + ks * 32 + lg8);
         o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o, 0, 0, 0);
       }
     };
-    bf16x8 vb1[16];
-    if (vtotal > 16) {  // the other sixteen pieces, in flight while the first are multiplied
+    bf16x8 vb1[8];
+    if (vtotal > 8) {  // the other eight pieces, in flight while the first are multiplied
 #pragma unroll
-      for (int f0 = 0; f0 < 16; f0 += 8) {
-        if (16 + f0 < vtotal) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) vb1[f0 + i] = value_piece(16 + f0 + i);
-        }
-      }
+      for (int i = 0; i < 8; ++i) vb1[i] = value_piece(8 + i);
     }
 #pragma unroll
-    for (int f = 0; f < 16; ++f) weigh(f, vb0[f], acc[f >> 1]);
-    if (vtotal > 16) {
+    for (int f = 0; f < 8; ++f) weigh(f, vb0[f], acc[f >> 1]);
+    if (vtotal > 8) {
 #pragma unroll
-      for (int f = 16; f < 32; ++f) weigh(f, vb1[f - 16], acc[f >> 1]);
+      for (int f = 8; f < 16; ++f) weigh(f, vb1[f - 8], acc[f >> 1]);
     }
   }
   __syncthreads();
   bf16* out = reinterpret_cast<bf16*>(a.out);
   const size_t pbase = ((size_t)item * splits + split) * tq;
 #pragma unroll
-  for (int t = 0; t < AMM_TILES; ++t) {
-    if (t >= KV * CTW) break;
-    const int c = t / CTW, ct = wave + AM_WAVES * (t - c * CTW);
+  for (int t = 0; t < AMM_TILES / 2; ++t) {
+    if (t >= KVh * CTW) break;
+    const int c = 2 * (t / CTW) + half, ct = wave + 4 * (t % CTW);
     if (ct >= CT) continue;
     const int d = ct * 16 + lr;
 #pragma unroll
@@ -596,7 +594,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_headmix_mfma_kernel(MixArgs a
     }
   }
   if (splits > 1)
-    for (int i = tid; i < tq * H; i += AM_THREADS) {
+    for (int i = tid; i < tq * H; i += AMM_THREADS) {
       part_ml[(pbase * H + i) * 2] = row_m[i];
       part_ml[(pbase * H + i) * 2 + 1] = row_l[i];
     }
@@ -673,7 +671,7 @@ extern "C" int as_attn_headmix_mfma(const void* q, const void* k_pages, const vo
         return AS_LAUNCH_FAILED;                                                                                   \
       raised = true;                                                                                               \
     }                                                                                                              \
-    attn_headmix_mfma_kernel<DS><<<dim3(num_items, splits), AM_THREADS, lds, stream>>>(a, tq, single, splits,      \
+    attn_headmix_mfma_kernel<DS><<<dim3(num_items, splits), AMM_THREADS, lds, stream>>>(a, tq, single, splits,      \
                                                                                        part_o, part_ml);           \
     break;                                                                                                         \
   }
