@@ -416,8 +416,8 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
     if (tid < AM_KC) pages[tid] = slot_valid ? table[lp] : 0;
     __syncthreads();
     // ---- phase 1: scores of this wave's 16 keys for every kv head ---------------------------------
-    // (kv head, 32 coordinates) pieces of the wave's keys, sixteen at a time: all of them are asked for before the
-    // first product (a wait for memory per sixteen), in batches of 8 so that small models ask for no more than they have
+    // (kv head, 32 coordinates) pieces of the wave's keys, eight at a time: all eight are asked for before the first
+    // product (a wait for memory per eight)
     // what a lane adds to its addresses, hidden from the compiler at every chunk: it would otherwise keep every
     // piece's address in registers of its own for the whole kernel (a hundred of them) and spill the products' operands
     int lg8 = lg * 8, lrv = lr;
@@ -429,22 +429,17 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
     {
       floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int h0 = 0; h0 < AMM_PIECES / 2; h0 += 16) {
+      for (int h0 = 0; h0 < AMM_PIECES / 2; h0 += 8) {
         if (h0 >= total) break;
-        bf16x8 kb[16];
+        bf16x8 kb[8];
 #pragma unroll
-        for (int f0 = 0; f0 < 16; f0 += 8) {
-          if (h0 + f0 < total) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-              const int f = min(h0 + f0 + i, total - 1);
-              const int c = 2 * (f / DS) + half, d0 = (f % DS) * 32;
-              kb[f0 + i] = *reinterpret_cast<const bf16x8*>(kp + kbase + (size_t)c * bs * D + d0 + lg8);
-            }
-          }
+        for (int i = 0; i < 8; ++i) {
+          const int f = min(h0 + i, total - 1);
+          const int c = 2 * (f / DS) + half, d0 = (f % DS) * 32;
+          kb[i] = *reinterpret_cast<const bf16x8*>(kp + kbase + (size_t)c * bs * D + d0 + lg8);
         }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < 8; ++i) {
           const int f = h0 + i;
           if (f < total) {
             const int c = 2 * (f / DS) + half, ds = f % DS;
@@ -484,7 +479,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
       float mixed[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) mixed[j] = 0.f;
-#pragma unroll 4
+#pragma unroll 2
       for (int g = 0; g < H; ++g) {
         const float r = sraw[((size_t)g * tq + qi) * AM_KC + lane];
         const float4 t0 = *reinterpret_cast<const float4*>(mixT + g * H8 + h0);
