@@ -492,43 +492,47 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
       const int ipos = p0 + qi;
       const bool seen = slot_valid && qi < count && jpos <= ipos &&
                         (a.window <= 0 || ipos - jpos < a.window || jpos < a.keep_first);
-      // the eight rows' maxima and sums side by side, so that their lane swaps overlap
-      float mx[8], m_old[8], m_new[8], pr[8], sm[8], al[8];
+      // four rows' maxima and sums side by side at a time, so that their lane swaps overlap
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        mixed[j] = seen ? mixed[j] : -INFINITY;
-        mx[j] = mixed[j];
-        m_old[j] = h0 + j < H ? row_m[qi * H + h0 + j] : -INFINITY;
-      }
+      for (int j0 = 0; j0 < 8; j0 += 4) {
+        if (h0 + j0 >= H) break;
+        float sv[4], mx[4], m_old[4], pr[4], al[4];
 #pragma unroll
-      for (int off = WAVE / 2; off > 0; off >>= 1)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], off, WAVE));
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        m_new[j] = fmaxf(m_old[j], mx[j]);
-        pr[j] = 0.f;
-        al[j] = 1.f;
-        if (m_new[j] > -INFINITY) {
-          pr[j] = seen ? expf(mixed[j] - m_new[j]) : 0.f;
-          al[j] = m_old[j] > -INFINITY ? expf(m_old[j] - m_new[j]) : 0.f;
+        for (int j = 0; j < 4; ++j) {
+          sv[j] = seen ? mixed[j0 + j] : -INFINITY;
+          mx[j] = sv[j];
+          m_old[j] = h0 + j0 + j < H ? row_m[qi * H + h0 + j0 + j] : -INFINITY;
         }
-        sm[j] = pr[j];
-      }
 #pragma unroll
-      for (int off = WAVE / 2; off > 0; off >>= 1)
+        for (int off = WAVE / 2; off > 0; off >>= 1)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) sm[j] += __shfl_xor(sm[j], off, WAVE);
+          for (int j = 0; j < 4; ++j) mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], off, WAVE));
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int h = h0 + j;
-        if (h >= H) break;
-        const int rr = qi * H + h;
-        pb[((size_t)h * tq + qi) * AM_KC + lane] = (bf16)pr[j];
-        if (lane == 0) {
-          row_m[rr] = m_new[j];
-          row_l[rr] = row_l[rr] * al[j] + sm[j];
-          row_a[rr] = al[j];
+        for (int j = 0; j < 4; ++j) {
+          mx[j] = fmaxf(m_old[j], mx[j]);  // the new maximum
+          pr[j] = 0.f;
+          al[j] = 1.f;
+          if (mx[j] > -INFINITY) {
+            pr[j] = seen ? expf(sv[j] - mx[j]) : 0.f;
+            al[j] = m_old[j] > -INFINITY ? expf(m_old[j] - mx[j]) : 0.f;
+          }
+          sv[j] = pr[j];  // to be summed over the lanes
+        }
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) sv[j] += __shfl_xor(sv[j], off, WAVE);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int h = h0 + j0 + j;
+          if (h >= H) break;
+          const int rr = qi * H + h;
+          pb[((size_t)h * tq + qi) * AM_KC + lane] = (bf16)pr[j];
+          if (lane == 0) {
+            row_m[rr] = mx[j];
+            row_l[rr] = row_l[rr] * al[j] + sv[j];
+            row_a[rr] = al[j];
+          }
         }
       }
     }
@@ -553,16 +557,13 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
         o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o, 0, 0, 0);
       }
     };
-    bf16x8 vb1[8];
-    if (vtotal > 8) {  // the other eight pieces, in flight while the first are multiplied
-#pragma unroll
-      for (int i = 0; i < 8; ++i) vb1[i] = value_piece(8 + i);
-    }
 #pragma unroll
     for (int f = 0; f < 8; ++f) weigh(f, vb0[f], acc[f >> 1]);
-    if (vtotal > 8) {
+    if (vtotal > 8) {  // the other eight pieces (a model of many kv heads or wide heads)
 #pragma unroll
-      for (int f = 8; f < 16; ++f) weigh(f, vb1[f - 8], acc[f >> 1]);
+      for (int i = 0; i < 8; ++i) vb0[i] = value_piece(8 + i);
+#pragma unroll
+      for (int f = 8; f < 16; ++f) weigh(f, vb0[f - 8], acc[f >> 1]);
     }
   }
   __syncthreads();
