@@ -638,7 +638,7 @@ static size_t headmix_mfma_lds(int H, int D, int tq) {
 static bool headmix_mfma_takes(int H, int KV, int D, int bs, int tq) {
   if (H <= 0 || KV <= 0 || H % KV || H > 64 || tq < 1) return false;
   const int group = H / KV;
-  if (group * tq > 16) return false;
+  if (group * tq > 16 || (group & (group - 1))) return false;  // the rows of a tile are cut by shifts
   if (D % 32 || D > 256 || D == 160 || D == 224 || KV * ((D + 63) / 64) > AMM_TILES) return false;
   if (bs % 8 || bs > AM_KC || AM_KC % bs) return false;
   return headmix_mfma_lds(H, D, tq) <= (size_t)(128 << 10);

@@ -1165,6 +1165,8 @@ def attn_headmix_mfma_takes(dtype, H: int, KV: int, D: int, block_size: int, til
     pages of 8, 16, 32 or 64 tokens."""
     if dtype != BF16 or H < 1 or KV < 1 or H % KV or H > 64 or tile < 1 or (H // KV) * tile > 16:
         return False
+    if (H // KV) & (H // KV - 1):  # 1, 2, 4, 8 or 16 query heads to a kv head: the rows of a tile are cut by shifts
+        return False
     if D not in (32, 64, 96, 128, 192, 256) or KV * -(-D // 64) > HEADMIX_MFMA_TILES:
         return False
     if block_size % 8 or block_size > HEADMIX_KEYS or HEADMIX_KEYS % block_size:

@@ -300,7 +300,8 @@ def attend(q, kp, vp, table, mix, scale, window, keep_first, dtype, tile, single
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 6, 24, 8), (18, 1, 8, 4), (16, 2, 64, 64), (3, 1, 40, 16), (32, 4, 128, 16),
-                                   (8, 2, 32, 8), (4, 4, 64, 32), (16, 1, 32, 16), (4, 4, 256, 16), (32, 8, 128, 4), (5, 5, 96, 16)])
+                                   (8, 2, 32, 8), (4, 4, 64, 32), (16, 1, 32, 16), (4, 4, 256, 16), (32, 8, 128, 4), (5, 5, 96, 16),
+                                   (6, 2, 64, 16), (3, 1, 64, 8), (12, 1, 32, 16)])
 def test_mixed_heads_attention_kernel(shape, dtype):
     """Random queries, keys and values over pages in a random order, a window of 37 with 5 kept tokens, a window of
     one, and none: in tiles, as single tokens, and both in one sequence.  In bfloat16 the shapes with heads of a
