@@ -77,25 +77,23 @@ __global__ __launch_bounds__(1024) void moe_route_table_kernel(const int* __rest
 // ---- a router that scores every expert ---------------------------------------------------------------
 // z = router h in fp32 (router [experts, K], h [T, K], both T-typed), s = sigmoid(z); a token's `top` experts are
 // those with the largest s (of equal ones the lower number first); their weights are s / (sum of the chosen + 1e-20).
-// pair_expert, pair_weight [T * top].  A workgroup per token: its waves take the experts in turn, a lane 16 bytes of
-// the router's row and of the token's at a time (the rows stream once, coalesced), the sums meet by lane swaps and the
-// scores in LDS, where the first wave makes the choice.
+// pair_expert, pair_weight [T * top].  A workgroup per token: its waves take the experts four at a time, a lane 16 bytes
+// of the token's row and of the four router rows at a time (the rows stream once, coalesced), the sums meet by lane swaps
+// and the scores in LDS, where the first wave makes the choice.
 template <typename T> struct RoutePiece;
 template <> struct RoutePiece<float> {
   static constexpr int N = 4;
-  static __device__ __forceinline__ float dot(const float* a, const float* b) {
-    const float4 x = *reinterpret_cast<const float4*>(a), y = *reinterpret_cast<const float4*>(b);
-    return fmaf(x.w, y.w, fmaf(x.z, y.z, fmaf(x.y, y.y, x.x * y.x)));
+  static __device__ __forceinline__ void load(const float* p, float* v) {
+    const float4 x = *reinterpret_cast<const float4*>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
   }
 };
 template <> struct RoutePiece<bf16> {
   static constexpr int N = 8;
-  static __device__ __forceinline__ float dot(const bf16* a, const bf16* b) {
-    const bf16x8 x = *reinterpret_cast<const bf16x8*>(a), y = *reinterpret_cast<const bf16x8*>(b);
-    float s = 0.f;
+  static __device__ __forceinline__ void load(const bf16* p, float* v) {
+    const bf16x8 x = *reinterpret_cast<const bf16x8*>(p);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) s = fmaf((float)x[i], (float)y[i], s);
-    return s;
+    for (int i = 0; i < 8; ++i) v[i] = (float)x[i];
   }
 };
 
@@ -110,16 +108,33 @@ __global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(const T* __restr
   const int t = blockIdx.x;
   const T* row = h + (size_t)t * K;
   const bool whole = K % N == 0;  // rows start on 16 bytes
-  for (int e = wave; e < experts; e += 4) {
-    const T* wr = router + (size_t)e * K;
-    float z = 0.f;
+  // a wave takes four experts at a time: the token's piece is loaded once for the four rows' pieces, and four
+  // rows' loads are in flight together
+  for (int e0 = wave * 4; e0 < experts; e0 += 16) {
+    float z[4] = {0.f, 0.f, 0.f, 0.f};
     if (whole) {
-      for (int k = lane * N; k < K; k += WAVE * N) z += RoutePiece<T>::dot(row + k, wr + k);
+      for (int k = lane * N; k < K; k += WAVE * N) {
+        float hv[N], wv[4][N];
+        RoutePiece<T>::load(row + k, hv);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) RoutePiece<T>::load(router + (size_t)min(e0 + j, experts - 1) * K + k, wv[j]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int i = 0; i < N; ++i) z[j] = fmaf(hv[i], wv[j][i], z[j]);
+      }
     } else {
-      for (int k = lane; k < K; k += WAVE) z = fmaf(to_f32(row[k]), to_f32(wr[k]), z);
+      for (int k = lane; k < K; k += WAVE) {
+        const float hv = to_f32(row[k]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) z[j] = fmaf(hv, to_f32(router[(size_t)min(e0 + j, experts - 1) * K + k]), z[j]);
+      }
     }
-    z = wave_sum(z);
-    if (lane == 0) scores[e] = 1.0f / (1.0f + expf(-z));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float zs = wave_sum(z[j]);
+      if (lane == 0 && e0 + j < experts) scores[e0 + j] = 1.0f / (1.0f + expf(-zs));
+    }
   }
   __syncthreads();
   if (wave) return;

@@ -197,7 +197,7 @@ def koravik_config(width: int, layers: int, vocab: int):
     mlp = {"kind": "moe", "expert": {"ff": 3 * width // 4}, "router": {"experts": 16, "top": 2}, "shared": {"ff": 3 * width // 2}}
     distinct = max(3, layers - 2)
     return KoravikConfig.from_dict({"architecture": "Koravik", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
-                                    "residual_mult": 0.7, "logit_scale": 0.5,
+                                    "residual_mult": 0.8, "logit_scale": 1.0,
                                     "layers": [{"type": "attention", "mixer": mixer, "mlp": mlp} for _ in range(distinct)],
                                     "loop": {"start": 1, "stop": 3, "times": 2}})  # fmt: skip
 

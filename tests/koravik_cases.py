@@ -37,7 +37,7 @@ CASES = {
     "plain_order": {
         "architecture": "Koravik", "vocab": 128, "width": 64, "norm": {"eps": 1e-5}, "residual_mult": 1.0, "logit_scale": 0.25,
         "layers": [
-            {"type": "attention", "mixer": _attn(4, 4, 32, 0.2, 32, 250000.0, 1000, 0), "mlp": _moe(16, 3, 3, shared=16)},
+            {"type": "attention", "mixer": _attn(4, 4, 32, 0.2, 32, 300000.0, 1000, 0), "mlp": _moe(16, 3, 3, shared=16)},
             {"type": "attention", "mixer": _attn(2, 1, 12, 0.5, 6, 50.0, 1, 2), "mlp": _moe(8, 2, 1, shared=8)},
             {"type": "attention", "mixer": _attn(2, 2, 8, 0.35, 0, 10.0, 6, 1), "mlp": None},
         ],

@@ -543,7 +543,7 @@ def test_router_takes_the_lower_number_of_equal_scores():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("width", [48, 320, 2056])
+@pytest.mark.parametrize("width", [48, 344, 2056])
 def test_gated_sum_norm_and_join(width, dtype):
     """x += m sigmoid(g + b) y in 32 bits, the norm of the sum, rows picked out, the stream left alone where asked,
     and the sum beside another stream as a product's input."""
@@ -555,23 +555,23 @@ def test_gated_sum_norm_and_join(width, dtype):
     y, gate = bf(torch.randn(T, width, generator=gen)), bf(torch.randn(T, width + 24, generator=gen))
     bias, gain = bf(torch.randn(width, generator=gen)), bf(1 + 0.1 * torch.randn(width, generator=gen))
     other = torch.randn(T, width, generator=gen)
-    want_x = x.double() + 0.7 * torch.sigmoid(gate[:, 24:].double() + bias.double()) * y.double()
+    want_x = x.double() + 0.6 * torch.sigmoid(gate[:, 24:].double() + bias.double()) * y.double()
     want_h = plain.rms_norm(want_x, gain.double(), 1e-5)
     tol = 2e-6 if dtype == "float32" else 1e-2
     dev = lambda a, kind=t: a.to(DEV).to(kind).contiguous()  # noqa: E731
     xs = dev(x, torch.float32)
     out = torch.empty((T, width), dtype=t, device=DEV)
-    ops.gated_add_norm(xs, dev(y), dev(gate), 24, dev(bias), 0.7, dev(gain), 1e-5, out)
+    ops.gated_add_norm(xs, dev(y), dev(gate), 24, dev(bias), 0.6, dev(gain), 1e-5, out)
     assert (xs.cpu().double() - want_x).abs().max() <= 2e-6 * float(want_x.abs().max())
     assert (out.float().cpu().double() - want_h).abs().max() <= tol * float(want_h.abs().max())
     rows = torch.tensor([11, 2, 2, 0], dtype=torch.int32, device=DEV)
     xs = dev(x, torch.float32)
     picked = torch.empty((4, width), dtype=t, device=DEV)
-    ops.gated_add_norm(xs, dev(y), dev(gate), 24, dev(bias), 0.7, dev(gain), 1e-5, picked, rows=rows, update_x=False)
+    ops.gated_add_norm(xs, dev(y), dev(gate), 24, dev(bias), 0.6, dev(gain), 1e-5, picked, rows=rows, update_x=False)
     assert torch.equal(xs.cpu(), x) and (picked.float().cpu().double() - want_h[[11, 2, 2, 0]]).abs().max() <= tol * float(want_h.abs().max())
     xs = dev(x, torch.float32)
     join = torch.empty((T, 2 * width), dtype=t, device=DEV)
-    ops.gated_add_norm(xs, dev(y), dev(gate), 24, dev(bias), 0.7, None, 0.0, None, other=dev(other, torch.float32), join=join)
+    ops.gated_add_norm(xs, dev(y), dev(gate), 24, dev(bias), 0.6, None, 0.0, None, other=dev(other, torch.float32), join=join)
     assert (join[:, :width].float().cpu().double() - want_x).abs().max() <= tol * float(want_x.abs().max())
     assert (join[:, width:].float().cpu() - other).abs().max() <= tol * float(other.abs().max())
     plain_norm = torch.empty((T, width), dtype=torch.float32, device=DEV)  # a norm whose result is a stream: 32 bits out
