@@ -328,6 +328,33 @@ extern "C" int as_attn_headmix(const void* q, const void* k_pages, const void* v
 // `splits` workgroups share an item's chunks and leave unnormalised outputs, maxima and sums for the merge kernel.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// Maxima and sums over all 64 lanes, in every lane, without LDS: within a row of 16 lanes by DPP moves (lane ^ 1,
+// lane ^ 2, the mirror image within eight lanes and within sixteen), then over the four rows by v_permlane16_swap /
+// v_permlane32_swap (with both operands equal they hand every lane the other rows' values).
+template <int CTRL> __device__ __forceinline__ float amm_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float amm_all_max(float v) {
+  v = fmaxf(v, amm_dpp<0xB1>(v));   // quad_perm [1, 0, 3, 2]
+  v = fmaxf(v, amm_dpp<0x4E>(v));   // quad_perm [2, 3, 0, 1]
+  v = fmaxf(v, amm_dpp<0x141>(v));  // row_half_mirror
+  v = fmaxf(v, amm_dpp<0x140>(v));  // row_mirror
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float amm_all_sum(float v) {
+  v += amm_dpp<0xB1>(v);
+  v += amm_dpp<0x4E>(v);
+  v += amm_dpp<0x141>(v);
+  v += amm_dpp<0x140>(v);
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
 #define AMM_TILES 16  // output tiles (kv head, column tile) a wave keeps: KV * ceil(D / 64) at most
 #define AMM_THREADS 512  // eight waves, two to a SIMD
 #define AMM_PIECES 32  // 16-byte pieces of keys, and of values, that a lane asks for per chunk: KV * D / 32 at most
@@ -492,7 +519,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
       const int ipos = p0 + qi;
       const bool seen = slot_valid && qi < count && jpos <= ipos &&
                         (a.window <= 0 || ipos - jpos < a.window || jpos < a.keep_first);
-      // four rows' maxima and sums side by side at a time, so that their lane swaps overlap
+      // four rows' maxima and sums at a time, by lane swaps that do not pass through LDS
 #pragma unroll
       for (int j0 = 0; j0 < 8; j0 += 4) {
         if (h0 + j0 >= H) break;
@@ -504,9 +531,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
           m_old[j] = h0 + j0 + j < H ? row_m[qi * H + h0 + j0 + j] : -INFINITY;
         }
 #pragma unroll
-        for (int off = WAVE / 2; off > 0; off >>= 1)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], off, WAVE));
+        for (int j = 0; j < 4; ++j) mx[j] = amm_all_max(mx[j]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           mx[j] = fmaxf(m_old[j], mx[j]);  // the new maximum
@@ -519,9 +544,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
           sv[j] = pr[j];  // to be summed over the lanes
         }
 #pragma unroll
-        for (int off = WAVE / 2; off > 0; off >>= 1)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) sv[j] += __shfl_xor(sv[j], off, WAVE);
+        for (int j = 0; j < 4; ++j) sv[j] = amm_all_sum(sv[j]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int h = h0 + j0 + j;
