@@ -302,28 +302,30 @@ class KoravikAttention:
     scale: float  # multiplies q.k
     rot_dims: int  # coordinates of a head that turn with the position
     rot_base: float
-    window: int  # keys a position sees, itself included
+    window: int  # keys a position sees, itself included; 0: all
     keep_first: int  # the sequence's first tokens, which stay visible behind the window
 
     @classmethod
     def from_dict(cls, raw: dict, where: str) -> "KoravikAttention":
-        rot, mask = _need(raw, "rot", where), _need(raw, "mask", where)
+        rot, mask = raw.get("rot") or {}, raw.get("mask") or {}  # neither: nothing turns, every earlier key is seen
         return cls(
             heads=int(_need(raw, "heads", where)),
             kv_heads=int(_need(raw, "kv_heads", where)),
             dim=int(_need(raw, "dim", where)),
             vdim=int(raw.get("vdim", raw.get("dim", 0))),
             scale=float(_need(raw, "scale", where)),
-            rot_dims=int(_need(rot, "dims", where + "rot.")),
-            rot_base=float(_need(rot, "base", where + "rot.")),
-            window=int(_need(mask, "size", where + "mask.")),
+            rot_dims=int(rot.get("dims", 0)),
+            rot_base=float(_need(rot, "base", where + "rot.")) if rot.get("dims") else 1.0,
+            window=int(mask.get("size", 0)),
             keep_first=int(mask.get("keep_first", 0)),
         )
 
     def to_dict(self) -> dict:
-        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale,
-                "rot": {"dims": self.rot_dims, "base": self.rot_base},
-                "mask": {"size": self.window, "keep_first": self.keep_first}}  # fmt: skip
+        raw = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale,
+               "rot": {"dims": self.rot_dims, "base": self.rot_base}}  # fmt: skip
+        if self.window:
+            raw["mask"] = {"size": self.window, "keep_first": self.keep_first}
+        return raw
 
 
 @dataclass(frozen=True)
@@ -426,8 +428,8 @@ class KoravikConfig:
                 raise ConfigError(f"layers[{i}]: the values are the keys, so vdim {m.vdim} must equal dim {m.dim}")
             if m.rot_dims < 0 or m.rot_dims % 2 or m.rot_dims > m.dim or not m.rot_base > 0:
                 raise ConfigError(f"layers[{i}]: rot.dims must be even and at most dim, rot.base positive")
-            if m.window < 1 or m.keep_first < 0:
-                raise ConfigError(f"layers[{i}]: mask.size must be positive and mask.keep_first not negative")
+            if m.window < 0 or m.keep_first < 0:
+                raise ConfigError(f"layers[{i}]: mask.size and mask.keep_first must not be negative")
             f = layer.mlp
             if f is not None and (f.ff < 1 or f.shared_ff < 0 or not 1 <= f.top <= f.experts):
                 raise ConfigError(f"layers[{i}].mlp: sizes must be positive and top at most the number of experts")

@@ -70,10 +70,11 @@ def attention(h, w, p, m, round_to=_id):
     k = round_to(h @ w[p + "k"].T).view(T, G, D)
     v = k  # the keys as projected are the values
     pos = torch.arange(T)
-    if m["rot"]["dims"]:
-        q = round_to(turn_half(q, pos, m["rot"]["dims"], m["rot"]["base"]))
-        k = round_to(turn_half(k, pos, m["rot"]["dims"], m["rot"]["base"]))
-    o = mixed_softmax_attention(q, k, v, w[p + "talk"], m["scale"], m["mask"]["size"], m["mask"].get("keep_first", 0))
+    rot, mask = m.get("rot") or {}, m.get("mask") or {}  # neither: nothing turns, every earlier key is seen
+    if rot.get("dims"):
+        q = round_to(turn_half(q, pos, rot["dims"], rot["base"]))
+        k = round_to(turn_half(k, pos, rot["dims"], rot["base"]))
+    o = mixed_softmax_attention(q, k, v, w[p + "talk"], m["scale"], mask.get("size") or T + 1, mask.get("keep_first", 0))
     return round_to(round_to(o).reshape(T, H * D) @ w[p + "o"].T)
 
 

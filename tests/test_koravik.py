@@ -72,7 +72,7 @@ def test_what_the_configuration_refuses():
         (lambda r: r["layers"][0]["mixer"]["rot"].update(dims=7), "rot.dims"),
         (lambda r: r["layers"][0]["mixer"]["rot"].update(dims=18), "rot.dims"),
         (lambda r: r["layers"][0]["mixer"].pop("scale"), "scale"),
-        (lambda r: r["layers"][0]["mixer"]["mask"].update(size=0), "mask.size"),
+        (lambda r: r["layers"][0]["mixer"]["mask"].update(size=-1), "mask.size"),
         (lambda r: r["layers"][1]["mixer"].update(kv_heads=2), "kv_heads"),
         (lambda r: r.update(loop={"start": 2, "stop": 5, "times": 2}), "loop"),
         (lambda r: r["layers"][0]["mlp"]["router"].update(top=6), "top"),
@@ -82,6 +82,19 @@ def test_what_the_configuration_refuses():
         change(bad)
         with pytest.raises(ConfigError, match=needle):
             KoravikConfig.from_dict(bad)
+
+
+def test_a_mixer_without_a_mask_or_a_rotation_sees_every_earlier_key_and_turns_nothing():
+    from atomserve_amd.config.model_config import KoravikConfig
+
+    raw = copy.deepcopy(CASES["wide_groups"])
+    raw["layers"][0]["mixer"].pop("mask")
+    raw["layers"][1]["mixer"].pop("rot")
+    config = KoravikConfig.from_dict(raw)
+    assert (config.layers[0].mixer.window, config.layers[0].mixer.keep_first, config.layers[1].mixer.rot_dims) == (0, 0, 0)
+    assert KoravikConfig.from_dict(config.to_dict()) == config
+    _, _, model = parts_of(raw)
+    assert model.cache_requests()[0].window == 0 and model.blocks[1].parts()["mixer"].position is None
 
 
 def test_a_layer_with_gated_sums_needs_parts_that_compute_their_gate():

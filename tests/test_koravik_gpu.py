@@ -128,6 +128,26 @@ def test_whole_decoded_in_portions_and_mixed(case, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_model_whose_mixers_name_no_mask_or_no_rotation(dtype):
+    """Without a mask a position sees every earlier key (nothing is given back), without a rotation nothing turns."""
+    raw = copy.deepcopy(CASES["wide_groups"])
+    raw["layers"][0]["mixer"].pop("mask")
+    raw["layers"][1]["mixer"].pop("rot")
+    weights = random_weights(raw, seed=12)
+    requests = {"a": rc.random_ids(raw["vocab"], 90, 6), "b": rc.random_ids(raw["vocab"], 33, 7)}
+    replay = make_replay(raw, weights, dtype, max_tokens=2 * 128, max_live=2)
+    refs, total = {}, Against()
+    for steps in (rc.whole("a", requests["a"]), rc.portions("a", requests["a"]), rc.mixed(requests, seed=5, max_live=2),
+                  rc.prefill_then_decode("b", requests["b"], tail=20)):  # fmt: skip
+        result = compare(replay, steps, requests, raw, weights, refs, dtype)
+        total.err += result.err
+        total.noise += result.noise
+        total.scale = max(total.scale, result.scale)
+    total.check(dtype, "no mask, no rotation")
+    assert replay.manager.num_free == replay.manager.num_blocks
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("block_size", [4, 8, 64])
 def test_pages_of_other_sizes(block_size, dtype):
     """Windows and kept tokens against pages of 4, 8 and 64 tokens: portions and a mixed batch."""
