@@ -257,6 +257,33 @@ def test_the_replay_tool_on_a_folder(tmp_path):
     assert (got1 - ref[[29]]).abs().max() <= 3e-5 * float(ref.abs().max())
 
 
+def test_the_command_line_generates_from_a_folder_and_from_random_weights(tmp_path, capsys):
+    """`atomserve FOLDER --prompt-ids ...` on a Koravik folder written here: the architecture is found by its name
+    in config.json, the weights by their names, and the greedy tokens are the plain model's; with
+    `--random-weights` the same configuration generates without a checkpoint."""
+    from safetensors.torch import save_file
+
+    from atomserve_amd.engine import cli
+
+    raw = CASES["all_looped"]
+    weights = random_weights(raw, seed=17)
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    save_file({k: v.bfloat16().contiguous() for k, v in weights.items()}, str(tmp_path / "model.safetensors"))
+    prompt = rc.random_ids(raw["vocab"], 21, 3)
+    common = ["--dtype", "fp32", "--prompt-ids", " ".join(map(str, prompt)), "--max-tokens", "5", "--temperature", "0",
+              "--ignore-eos", "--kv-mem-gb", "0.05", "--max-num-seqs", "2", "--max-batched-tokens", "16"]  # fmt: skip
+    assert cli.main([str(tmp_path), *common]) == 0
+    lines = [json.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
+    want, seq = [], list(prompt)
+    for _ in range(5):
+        want.append(int(plain.logits(raw, weights, seq)[-1].argmax()))
+        seq.append(want[-1])
+    assert lines[-1]["output_ids"] == want
+    assert cli.main([str(tmp_path), "--random-weights", "3", *common]) == 0
+    lines = [json.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
+    assert len(lines[-1]["output_ids"]) == 5
+
+
 # ---- each mechanism alone ---------------------------------------------------------------------------------
 
 
