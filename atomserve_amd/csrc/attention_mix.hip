@@ -370,14 +370,17 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
   constexpr int D = 32 * DS, CT = 2 * DS, CTW = (CT + 3) / 4;  // column tiles of a head, and of a wave at most
   const int H = a.H, KV = a.KV, bs = a.bs, group = H / KV, gshift = __builtin_ctz(group), gmask = group - 1;
   const int H8 = (H + 7) & ~7, HB = H8 >> 3;
-  float* sraw = reinterpret_cast<float*>(lds_raw);             // [H][tq][64]
-  float* mixT = sraw + (size_t)H * tq * AM_KC;                 // [H][H8]: mixT[g][h] = mix[h][g]
+  // rows of scores, weights and queries are a little longer than what they hold, so that the 16 rows a product's
+  // operand is read from (and the 4 a product's result is written to) lie in different banks
+  constexpr int SROW = AM_KC + 1, PROW = AM_KC + 8, QROW = D + 8;
+  float* sraw = reinterpret_cast<float*>(lds_raw);             // [H][tq][SROW]
+  float* mixT = sraw + (((size_t)H * tq * SROW + 3) & ~(size_t)3);  // [H][H8]: mixT[g][h] = mix[h][g], read 16 bytes at a time
   float* row_m = mixT + H * H8;
   float* row_l = row_m + tq * H;
   float* row_a = row_l + tq * H;
   int* pages = reinterpret_cast<int*>(row_a + tq * H);         // [64]
-  bf16* pb = reinterpret_cast<bf16*>((reinterpret_cast<uintptr_t>(pages + AM_KC) + 15) & ~(uintptr_t)15);  // [H][tq][64]
-  bf16* qs = pb + (size_t)H * tq * AM_KC;                      // [tq][H][D]
+  bf16* pb = reinterpret_cast<bf16*>((reinterpret_cast<uintptr_t>(pages + AM_KC) + 15) & ~(uintptr_t)15);  // [H][tq][PROW]
+  bf16* qs = pb + (size_t)H * tq * PROW;                       // [tq][H][QROW]
 
   // eight waves: wave & 3 says which 16 of a chunk's keys (scores) and which column tiles (values) a wave takes,
   // wave >> 2 which half of the kv heads (the even or the odd ones); two waves share a SIMD and fill each other's waits
@@ -413,13 +416,13 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
   const int ch0 = split * cps, ch1 = min(chunks, ch0 + cps);
 
   for (int i = tid * 8; i < tq * HD; i += AMM_THREADS * 8) {  // 16 bytes a thread: D % 8 == 0
-    const int qi = i / HD;
+    const int qi = i / HD, rest = i - qi * HD, h = rest / D, d = rest - h * D;
     bf16x8 v;
-    if (qi < count) v = *reinterpret_cast<const bf16x8*>(q + (size_t)(first + qi) * HD + (i - qi * HD));
+    if (qi < count) v = *reinterpret_cast<const bf16x8*>(q + (size_t)(first + qi) * HD + rest);
     else
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = (bf16)0.f;
-    *reinterpret_cast<bf16x8*>(qs + i) = v;
+    *reinterpret_cast<bf16x8*>(qs + ((size_t)qi * H + h) * QROW + d) = v;
   }
   for (int i = tid; i < H * H8; i += AMM_THREADS) {
     const int g = i / H8, h = i - g * H8;
@@ -452,7 +455,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
     const int slot = 16 * wave + lrv;
     const size_t kbase = ((size_t)pages[slot] * KV * bs + slot % bs) * D;
     const int total = KVh * DS;
-    const size_t q_at = a_valid ? ((size_t)a_qi * H + a_g) * D : 0;  // rows that stand for nothing read row 0 (and are not stored)
+    const size_t q_at = a_valid ? ((size_t)a_qi * H + a_g) * QROW : 0;  // rows that stand for nothing read row 0 (and are not stored)
     {
       floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -470,7 +473,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
           const int f = h0 + i;
           if (f < total) {
             const int c = 2 * (f / DS) + half, ds = f % DS;
-            const bf16x8 qa = *reinterpret_cast<const bf16x8*>(qs + q_at + (size_t)c * group * D + ds * 32 + lg8);
+            const bf16x8 qa = *reinterpret_cast<const bf16x8*>(qs + q_at + (size_t)c * group * QROW + ds * 32 + lg8);
             if (ds == 0) sc = floatx4{0.f, 0.f, 0.f, 0.f};
             sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa, kb[i], sc, 0, 0, 0);
             if (ds == DS - 1) {
@@ -479,7 +482,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
                 const int rho = 4 * lg + r;
                 if (rho < rows_used) {
                   const int qi = rho >> gshift, g = rho & gmask;
-                  sraw[((size_t)(c * group + g) * tq + qi) * AM_KC + slot] = sc[r] * a.scale;
+                  sraw[((size_t)(c * group + g) * tq + qi) * SROW + slot] = sc[r] * a.scale;
                 }
               }
             }
@@ -508,7 +511,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
       for (int j = 0; j < 8; ++j) mixed[j] = 0.f;
 #pragma unroll 2
       for (int g = 0; g < H; ++g) {
-        const float r = sraw[((size_t)g * tq + qi) * AM_KC + lane];
+        const float r = sraw[((size_t)g * tq + qi) * SROW + lane];
         const float4 t0 = *reinterpret_cast<const float4*>(mixT + g * H8 + h0);
         const float4 t1 = *reinterpret_cast<const float4*>(mixT + g * H8 + h0 + 4);
         mixed[0] = fmaf(t0.x, r, mixed[0]); mixed[1] = fmaf(t0.y, r, mixed[1]);
@@ -550,7 +553,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
           const int h = h0 + j0 + j;
           if (h >= H) break;
           const int rr = qi * H + h;
-          pb[((size_t)h * tq + qi) * AM_KC + lane] = (bf16)pr[j];
+          pb[((size_t)h * tq + qi) * PROW + lane] = (bf16)pr[j];
           if (lane == 0) {
             row_m[rr] = mx[j];
             row_l[rr] = row_l[rr] * al[j] + sv[j];
@@ -561,7 +564,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
     }
     AMM_LDS_BARRIER();
     // ---- phase 3: weights times values ------------------------------------------------------------------
-    const size_t p_at = a_valid ? ((size_t)a_g * tq + a_qi) * AM_KC : 0;
+    const size_t p_at = a_valid ? ((size_t)a_g * tq + a_qi) * PROW : 0;
     auto weigh = [&](int f, const bf16x8& vb, floatx4& o) {  // f static: the tile's accumulator is a register
       const int t = f >> 1, ks = f & 1;
       const int c = 2 * (t / CTW) + half, ct = wave + 4 * (t % CTW);
@@ -576,7 +579,7 @@ __global__ __launch_bounds__(AMM_THREADS) void attn_headmix_mfma_kernel(MixArgs 
             }
           }
         }
-        const bf16x8 pa = *reinterpret_cast<const bf16x8*>(pb + p_at + (size_t)c * group * tq * AM_KC + ks * 32 + lg8);
+        const bf16x8 pa = *reinterpret_cast<const bf16x8*>(pb + p_at + (size_t)c * group * tq * PROW + ks * 32 + lg8);
         o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, o, 0, 0, 0);
       }
     };
@@ -653,8 +656,8 @@ __global__ __launch_bounds__(128) void attn_headmix_merge_kernel(const int* __re
 
 static size_t headmix_mfma_lds(int H, int D, int tq) {
   const int H8 = (H + 7) & ~7;
-  return ((size_t)H * tq * AM_KC + (size_t)H * H8 + 3 * (size_t)tq * H + AM_KC) * 4 + 16 +
-         ((size_t)H * tq * AM_KC + (size_t)tq * H * D) * 2;
+  return ((((size_t)H * tq * (AM_KC + 1) + 3) & ~(size_t)3) + (size_t)H * H8 + 3 * (size_t)tq * H + AM_KC) * 4 + 16 +
+         ((size_t)H * tq * (AM_KC + 8) + (size_t)tq * H * (D + 8)) * 2;  // rows padded against bank conflicts
 }
 
 // Whether the matrix-core kernel takes these sizes with items of up to `tq` queries (tq * group rows of a tile).

@@ -1156,7 +1156,8 @@ HEADMIX_MAX_SPLITS = 64
 
 def _headmix_mfma_lds(H: int, D: int, tq: int) -> int:
     h8 = -(-H // 8) * 8
-    return (H * tq * HEADMIX_KEYS + H * h8 + 3 * tq * H + HEADMIX_KEYS) * 4 + 16 + (H * tq * HEADMIX_KEYS + tq * H * D) * 2
+    scores = -(-H * tq * (HEADMIX_KEYS + 1) // 4) * 4  # rows a little longer than their 64 slots, against bank conflicts
+    return (scores + H * h8 + 3 * tq * H + HEADMIX_KEYS) * 4 + 16 + (H * tq * (HEADMIX_KEYS + 8) + tq * H * (D + 8)) * 2
 
 
 def attn_headmix_mfma_takes(dtype, H: int, KV: int, D: int, block_size: int, tile: int) -> bool:
